@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""SDDMM benchmark on one MI355X: GFLOP/s (2*nnz*K) on the FEM-banded fp32 K=32 shape.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--K K] [--strategy S]
+
+A step is one SDDMM over the whole sampling matrix with every operand already
+resident in HBM.  Prints ONE JSON line.  The result is validated against the CPU
+oracle before anything is timed; `cpu_baseline` times the reference CPU loop on
+the host cores of the same box in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """Reference CPU loop (1 thread, as the reference is serial) on the same inputs.
+    The whole workload is one sample when a run fits the budget, else a leading
+    block of rows.  Returns the dict for the JSON line plus an all-cores figure."""
+    from oracle import oracle as O
+    rowptr, col, sval = w.rowptr, w.col, w.sval
+    est = w.flops() / 1.0e9          # seconds at ~1 GFLOP/s, conservative
+    rows = w.M
+    if est > budget_s:
+        target = int(w.nnz * budget_s / est)
+        rows = max(1, int(np.searchsorted(rowptr, target)))
+    rp = np.ascontiguousarray(rowptr[: rows + 1])
+    nn = int(rp[-1])
+    cc, sv = np.ascontiguousarray(col[:nn]), np.ascontiguousarray(sval[:nn])
+    flops = 2.0 * nn * w.K
+    sample = "rows [0,%d) of %d: %d of %d entries, best of 3" % (rows, w.M, nn, w.nnz)
+    kind = "port"
+    best = None
+    if O.Ref.available():
+        # the reference's own CPUBasic<float>::run_csr compiled from its headers
+        kind = "reference"
+        coo_r = np.repeat(np.arange(rows, dtype=np.int32), np.diff(rp)).astype(np.int32)
+        best, _ = O.Ref().cpu_basic_csr_seconds(rows, w.N, coo_r, cc, sv, w.A[:rows], w.B, reps=3)
+    else:
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.sddmm_csr(rp, cc, sv, w.A, w.B, threads=1)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+    threads = O.max_threads()
+    allc = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.sddmm_csr(rp, cc, sv, w.A, w.B, threads=threads)
+        dt = time.perf_counter() - t0
+        allc = dt if allc is None else min(allc, dt)
+    return ({"value": flops / best / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": kind, "sample": sample},
+            {"value": flops / allc / 1e9, "unit": "GFLOP/s", "cores": threads, "kind": "port",
+             "sample": sample})
+
+
+def load_traffic(key):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
+    recorded by hand in profiles/traffic.json; None when not measured."""
+    p = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(p):
+        return None
+    try:
+        return json.load(open(p)).get(key, {}).get("bytes_per_launch")
+    except Exception:
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fem_banded")
+    ap.add_argument("--size", default="full", choices=["full", "small"])
+    ap.add_argument("--K", type=int, default=32)
+    ap.add_argument("--strategy", default="AUTO")
+    ap.add_argument("--include-plan", action="store_true", help="re-run the classifier inside every timed step")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip validation against the oracle")
+    args = ap.parse_args()
+
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        log("bench.py measures one GPU: SDDMM row panels are independent, there is no multi-GPU path "
+            "in this build (requested --gpus %d, WORLD_SIZE %d)." % (args.gpus, world))
+        sys.exit(2)
+
+    from dphpc_amd import capi, workloads
+
+    t0 = time.time()
+    w = workloads.make(args.workload, args.size, K=args.K)
+    log("workload %s: M=%d N=%d K=%d nnz=%d (%.1fs to generate)" % (w.name, w.M, w.N, w.K, w.nnz, time.time() - t0))
+    strategy = capi.STRATEGY_NAMES.index(args.strategy.upper())
+    bf16 = w.dtype == "bf16"
+
+    e = capi.Engine(0)
+    if bf16:
+        e.set_dense(w.A_bits, w.B_bits, capi.BF16)
+    else:
+        e.set_dense(w.A, w.B, capi.F32)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    e.plan(strategy)
+    plan_ms = e.stats().plan_ms
+
+    # ---- validate before timing ------------------------------------------------
+    validated = None
+    if not args.no_check:
+        from oracle import oracle as O
+        e.run()
+        got = e.values()
+        ref = O.sddmm_csr(w.rowptr, w.col, w.sval, w.A, w.B, threads=0)
+        _, mag = O.sddmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+        ok, worst, i = O.check_values(got, ref, mag=mag, rtol=1e-2 if bf16 and strategy == capi.MFMA_TILE else 1e-5)
+        if not ok:
+            log("VALIDATION FAILED: entry %d got %r ref %r (%.2f x tolerance)" % (i, got[i], ref[i], worst))
+            sys.exit(1)
+        validated = {"entries": int(len(got)), "worst_over_tol": round(worst, 4)}
+        log("validated %d entries against the CPU oracle (worst %.3f of tolerance)" % (len(got), worst))
+
+    # ---- timed region: W warm-up steps, then exactly K steps --------------------
+    for _ in range(args.warmup):
+        if args.include_plan:
+            e.plan(strategy)
+        e.launch()
+    e.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        if args.include_plan:
+            e.plan(strategy)
+        e.launch()
+    e.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+
+    # ---- per-launch device time from HIP events on the launch stream -----------
+    ev = e.time_runs(2, max(args.steps, 20), include_plan=args.include_plan)
+    ev_avg, ev_p50, ev_min = float(ev.mean()), float(np.median(ev)), float(ev.min())
+    st = e.stats()
+    flops, gathered = w.flops(), w.bytes_gathered()
+    achieved = gathered / (ev_avg * 1e-3) / 1e9
+
+    out = {
+        "metric": "SDDMM GFLOP/s (2*nnz*K), 1 MI355X, K=%d" % w.K,
+        "value": flops / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if bf16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": w.name, "size": args.size, "M": w.M, "N": w.N, "K": w.K, "nnz": w.nnz,
+                   "strategy": capi.STRATEGY_NAMES[st.strategy_used], "requested": args.strategy.upper(),
+                   "plan_in_step": bool(args.include_plan)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": load_traffic("%s_K%d_%s" % (w.name, w.K, "bf16" if bf16 else "f32"))},
+        "kernel_ms": {"avg": ev_avg, "p50": ev_p50, "min": ev_min, "launches_per_step": st.kernels_launched or 1},
+        "gflops_kernel": flops / (ev_avg * 1e-3) / 1e9,
+        "bytes_gathered": gathered,
+        "bytes_compulsory": w.bytes_compulsory(),
+        "plan_ms": plan_ms,
+        "validated": validated,
+    }
+    if not args.no_cpu:
+        base, allc = cpu_baseline(w)
+        out["cpu_baseline"] = base
+        out["cpu_allcores"] = allc
+    e.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

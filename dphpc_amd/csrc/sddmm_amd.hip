@@ -1,0 +1,673 @@
+// C ABI of the gfx950 SDDMM engine: context, operand upload, plan, launch.
+// See include/sddmm_amd.h for the contract of every entry point.
+#include "../../include/sddmm_amd.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "kernels_gather.h"
+#include "kernels_plan.h"
+
+using namespace sddmm;
+
+// ---------------------------------------------------------------------------
+struct sddmm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    char err[512] = {0};
+
+    // dense operands
+    int M = 0, N = 0, K = 0, dtype = SDDMM_F32;
+    bool have_dense = false;
+    void *dA = nullptr, *dB = nullptr;
+    bool own_dense = false;
+
+    // sparse operand
+    bool have_sparse = false, have_rowptr = false, own_sparse = false, from_coo = false;
+    int sM = 0, sN = 0;
+    int64_t nnz = 0;
+    int32_t *d_rowptr = nullptr, *d_col = nullptr, *d_rowidx = nullptr;
+    float *d_sval = nullptr, *dP = nullptr;
+    bool own_rowptr = false, own_rowidx = false;
+
+    // plan
+    bool planned = false;
+    int strategy = SDDMM_AUTO;       // resolved
+    int requested = SDDMM_AUTO;
+    PlanCounters *d_pc = nullptr;    // device counters
+    PlanCounters pc{};               // host copy
+    sddmm_stats stats{};
+};
+
+namespace {
+
+int fail(sddmm_ctx *c, int code, const char *fmt, ...) {
+    if (c) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(c->err, sizeof(c->err), fmt, ap);
+        va_end(ap);
+    }
+    return code;
+}
+
+#define HIP_TRY(c, call)                                                                         \
+    do {                                                                                         \
+        hipError_t e_ = (call);                                                                  \
+        if (e_ != hipSuccess)                                                                    \
+            return fail((c), SDDMM_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), \
+                        __FILE__, __LINE__);                                                     \
+    } while (0)
+
+#define ALLOC_TRY(c, ptr, bytes)                                                                 \
+    do {                                                                                         \
+        hipError_t e_ = hipMalloc((void **)&(ptr), (bytes) ? (bytes) : 16);                      \
+        if (e_ != hipSuccess) {                                                                  \
+            (ptr) = nullptr;                                                                     \
+            return fail((c), SDDMM_ERR_ALLOC, "hipMalloc(%zu bytes) failed: %s", (size_t)(bytes), \
+                        hipGetErrorString(e_));                                                  \
+        }                                                                                        \
+    } while (0)
+
+template <class T>
+void dfree(T *&p) {
+    if (p) (void)hipFree((void *)p);
+    p = nullptr;
+}
+
+void release_dense(sddmm_ctx *c) {
+    if (c->own_dense) { dfree(c->dA); dfree(c->dB); }
+    c->dA = c->dB = nullptr;
+    c->own_dense = false;
+    c->have_dense = false;
+    c->planned = false;
+}
+
+void release_sparse(sddmm_ctx *c) {
+    if (c->own_sparse) { dfree(c->d_col); dfree(c->d_sval); }
+    if (c->own_rowptr) dfree(c->d_rowptr);
+    if (c->own_rowidx) dfree(c->d_rowidx);
+    dfree(c->dP);
+    c->d_col = nullptr; c->d_sval = nullptr; c->d_rowptr = nullptr; c->d_rowidx = nullptr;
+    c->own_sparse = c->own_rowptr = c->own_rowidx = false;
+    c->have_sparse = c->have_rowptr = false;
+    c->from_coo = false;
+    c->planned = false;
+    c->nnz = 0;
+}
+
+size_t elem_size(int dtype) { return dtype == SDDMM_BF16 ? 2 : 4; }
+
+int grid_for(int64_t n, int block) { return (int)std::max<int64_t>(1, (n + block - 1) / block); }
+int grid_capped(int64_t n, int block, int cap = 16384) {
+    return (int)std::min<int64_t>(cap, std::max<int64_t>(1, (n + block - 1) / block));
+}
+
+int fetch_counters(sddmm_ctx *c) {
+    HIP_TRY(c, hipMemcpyAsync(&c->pc, c->d_pc, sizeof(PlanCounters), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+// power of two >= x, clamped to [1,64]
+int lanes_for(int units) {
+    int l = 1;
+    while (l < units && l < 64) l <<= 1;
+    return l;
+}
+
+// ---- kernel dispatch over (unit type, lanes per entry) -----------------------
+struct Shape {
+    int unit;   // 0: fp32 x4, 1: fp32 x1, 2: bf16 x8
+    int KU;     // units per row
+    int LPN;    // lanes per entry
+    bool single;
+};
+
+Shape shape_of(const sddmm_ctx *c) {
+    Shape s{};
+    if (c->dtype == SDDMM_BF16) { s.unit = 2; s.KU = c->K / 8; }
+    else if (c->K % 4 == 0) { s.unit = 0; s.KU = c->K / 4; }
+    else { s.unit = 1; s.KU = c->K; }
+    s.LPN = lanes_for(s.KU);
+    s.single = s.KU <= s.LPN;
+    return s;
+}
+
+template <class U, int LPN, bool SINGLE>
+void launch_flat_t(sddmm_ctx *c, int KU) {
+    const int64_t chunks = (c->nnz + WAVE - 1) / WAVE;
+    int cpw = (int)std::min<int64_t>(8, std::max<int64_t>(1, chunks / (WAVES_PER_BLOCK * 4096)));
+    const int64_t waves = (chunks + cpw - 1) / cpw;
+    const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    hipLaunchKernelGGL((k_flat<U, LPN, SINGLE>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                       (const typename U::T *)c->dA, (const typename U::T *)c->dB, KU, c->d_rowidx, c->d_col,
+                       c->d_sval, c->dP, c->nnz, cpw, nblocks);
+}
+
+template <class U, int LPN, bool SINGLE>
+void launch_row_wave_t(sddmm_ctx *c, int KU) {
+    const int64_t n_items = c->sM;
+    const int64_t nblocks = (n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    hipLaunchKernelGGL((k_row_wave<U, LPN, SINGLE>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                       (const typename U::T *)c->dA, (const typename U::T *)c->dB, KU, c->d_rowptr, c->d_col,
+                       c->d_sval, c->dP, (const RowItem *)nullptr, n_items, nblocks);
+}
+
+enum class Kern { Flat, RowWave };
+
+template <class U, int LPN, bool SINGLE>
+void launch_kind(sddmm_ctx *c, Kern k, int KU) {
+    if (k == Kern::Flat) launch_flat_t<U, LPN, SINGLE>(c, KU);
+    else launch_row_wave_t<U, LPN, SINGLE>(c, KU);
+}
+
+template <class U, int LPN>
+void launch_single(sddmm_ctx *c, Kern k, const Shape &s) {
+    if (s.single) launch_kind<U, LPN, true>(c, k, s.KU);
+    else launch_kind<U, LPN, false>(c, k, s.KU);
+}
+
+template <class U>
+void launch_lpn(sddmm_ctx *c, Kern k, const Shape &s) {
+    switch (s.LPN) {
+        case 1: launch_single<U, 1>(c, k, s); break;
+        case 2: launch_single<U, 2>(c, k, s); break;
+        case 4: launch_single<U, 4>(c, k, s); break;
+        case 8: launch_single<U, 8>(c, k, s); break;
+        case 16: launch_single<U, 16>(c, k, s); break;
+        case 32: launch_single<U, 32>(c, k, s); break;
+        default: launch_single<U, 64>(c, k, s); break;
+    }
+}
+
+void launch_gather(sddmm_ctx *c, Kern k) {
+    const Shape s = shape_of(c);
+    if (s.unit == 0) launch_lpn<UnitF32x4>(c, k, s);
+    else if (s.unit == 1) launch_lpn<UnitF32x1>(c, k, s);
+    else launch_lpn<UnitBF16x8>(c, k, s);
+}
+
+int ensure_rowidx(sddmm_ctx *c) {
+    if (c->d_rowidx) return SDDMM_OK;
+    ALLOC_TRY(c, c->d_rowidx, (size_t)c->nnz * sizeof(int32_t));
+    c->own_rowidx = true;
+    if (c->sM > 0 && c->nnz > 0)
+        hipLaunchKernelGGL(k_expand_rows, dim3(grid_for(c->sM, 256)), dim3(256), 0, c->stream, c->d_rowptr, c->sM,
+                           c->d_rowidx);
+    HIP_TRY(c, hipGetLastError());
+    return SDDMM_OK;
+}
+
+// Validate the device-resident CSR and gather row statistics.
+int validate_csr(sddmm_ctx *c) {
+    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+    if (c->sM > 0)
+        hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(c->sM, 256)), dim3(256), 0, c->stream, c->d_rowptr, c->sM,
+                           c->nnz, c->d_pc);
+    HIP_TRY(c, hipGetLastError());
+    int rc = fetch_counters(c);
+    if (rc) return rc;
+    if (c->pc.bad_pattern) return fail(c, SDDMM_ERR_PATTERN, "rowptr is not a valid CSR row pointer array");
+    // only now is it safe to walk col[0..nnz)
+    if (c->nnz > 0) {
+        hipLaunchKernelGGL(k_check_index, dim3(grid_capped(c->nnz, 256)), dim3(256), 0, c->stream, c->d_col, c->nnz,
+                           c->sN, c->d_pc);
+        HIP_TRY(c, hipGetLastError());
+        rc = fetch_counters(c);
+        if (rc) return rc;
+        if (c->pc.bad_pattern) return fail(c, SDDMM_ERR_PATTERN, "column index outside [0,N)");
+    }
+    return SDDMM_OK;
+}
+
+int check_dims(sddmm_ctx *c, int M, int N, int64_t nnz) {
+    if (M < 0 || N < 0 || nnz < 0) return fail(c, SDDMM_ERR_INVALID, "negative dimension");
+    if (nnz > 0 && (M == 0 || N == 0)) return fail(c, SDDMM_ERR_INVALID, "entries in an empty matrix");
+    if (nnz > (int64_t)INT32_MAX) return fail(c, SDDMM_ERR_INVALID, "nnz exceeds 32-bit row pointers");
+    return SDDMM_OK;
+}
+
+int enqueue_run(sddmm_ctx *c) {
+    if (c->nnz == 0) return SDDMM_OK;
+    switch (c->strategy) {
+        case SDDMM_FLAT: launch_gather(c, Kern::Flat); break;
+        case SDDMM_ROW_WAVE: launch_gather(c, Kern::RowWave); break;
+        case SDDMM_EXACT:
+            if (c->dtype == SDDMM_BF16)
+                hipLaunchKernelGGL(k_exact<true>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                                   c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
+            else
+                hipLaunchKernelGGL(k_exact<false>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                                   c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
+            break;
+        default: return fail(c, SDDMM_ERR_STATE, "no kernel for strategy %d", c->strategy);
+    }
+    HIP_TRY(c, hipGetLastError());
+    return SDDMM_OK;
+}
+
+int do_plan(sddmm_ctx *c, int strategy) {
+    int resolved = strategy;
+    const bool csr_ok = c->have_rowptr;
+    if (strategy == SDDMM_AUTO) {
+        if (!csr_ok) resolved = SDDMM_FLAT;
+        else {
+            const double avg = c->sM ? (double)c->nnz / (double)c->sM : 0.0;
+            const Shape s = shape_of(c);
+            // whole-row waves pay off once a typical row fills the 64-entry step and
+            // no single row dominates the run time
+            const bool balanced = (double)c->pc.max_len <= 64.0 * std::max(avg, 1.0);
+            resolved = (avg >= 2.0 * (WAVE / s.LPN) && balanced) ? SDDMM_ROW_WAVE : SDDMM_FLAT;
+        }
+    }
+    switch (resolved) {
+        case SDDMM_FLAT:
+        case SDDMM_EXACT: {
+            int rc = ensure_rowidx(c);
+            if (rc) return rc;
+            break;
+        }
+        case SDDMM_ROW_WAVE:
+            if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "ROW_WAVE needs row-sorted entries");
+            break;
+        case SDDMM_SHORT_ROWS:
+        case SDDMM_LDS_TILED:
+        case SDDMM_MFMA_TILE:
+            return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d is not available in this build", resolved);
+        default: return fail(c, SDDMM_ERR_INVALID, "unknown strategy %d", strategy);
+    }
+    c->requested = strategy;
+    c->strategy = resolved;
+    c->planned = true;
+    return SDDMM_OK;
+}
+
+void fill_model(sddmm_ctx *c) {
+    sddmm_stats &s = c->stats;
+    s.strategy_used = c->strategy;
+    s.nnz = c->nnz;
+    s.rows_nonempty = (int64_t)c->pc.rows_nonempty;
+    const double e = (double)elem_size(c->dtype);
+    s.flops = 2.0 * (double)c->nnz * (double)c->K;
+    s.bytes_gathered = 4.0 * ((double)c->sM + 1.0) + 12.0 * (double)c->nnz +
+                       e * (double)c->K * (double)s.rows_nonempty + e * (double)c->K * (double)c->nnz;
+}
+
+}  // namespace
+
+// ===========================================================================
+extern "C" {
+
+const char *sddmm_version(void) { return "sddmm_amd 0.1 (gfx950, wave64)"; }
+
+const char *sddmm_strerror(int code) {
+    switch (code) {
+        case SDDMM_OK: return "ok";
+        case SDDMM_ERR_INVALID: return "invalid argument";
+        case SDDMM_ERR_NULL: return "null pointer";
+        case SDDMM_ERR_STATE: return "operands or plan missing";
+        case SDDMM_ERR_ALLOC: return "allocation failed";
+        case SDDMM_ERR_HIP: return "HIP runtime error";
+        case SDDMM_ERR_UNSUPPORTED: return "strategy not applicable";
+        case SDDMM_ERR_NO_DEVICE: return "no usable HIP device";
+        case SDDMM_ERR_PATTERN: return "malformed sparse structure";
+        default: return "unknown error";
+    }
+}
+
+const char *sddmm_last_error(const sddmm_ctx *ctx) { return ctx ? ctx->err : ""; }
+
+int sddmm_create(sddmm_ctx **out, int device) {
+    if (!out) return SDDMM_ERR_NULL;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return SDDMM_ERR_NO_DEVICE;
+    if (device < 0 || device >= count) return SDDMM_ERR_INVALID;
+    if (hipSetDevice(device) != hipSuccess) return SDDMM_ERR_NO_DEVICE;
+    sddmm_ctx *c = new (std::nothrow) sddmm_ctx();
+    if (!c) return SDDMM_ERR_ALLOC;
+    c->device = device;
+    if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
+        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(PlanCounters)) != hipSuccess) {
+        sddmm_destroy(c);
+        return SDDMM_ERR_HIP;
+    }
+    *out = c;
+    return SDDMM_OK;
+}
+
+void sddmm_destroy(sddmm_ctx *c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    release_dense(c);
+    release_sparse(c);
+    dfree(c->d_pc);
+    if (c->ev0) (void)hipEventDestroy(c->ev0);
+    if (c->ev1) (void)hipEventDestroy(c->ev1);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+static int set_dense_common(sddmm_ctx *c, int M, int N, int K, const void *A, const void *B, int dtype,
+                            bool on_device) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    if (M < 0 || N < 0 || K < 1) return fail(c, SDDMM_ERR_INVALID, "need M,N >= 0 and K >= 1 (got %d,%d,%d)", M, N, K);
+    if (dtype != SDDMM_F32 && dtype != SDDMM_BF16) return fail(c, SDDMM_ERR_INVALID, "unknown dtype %d", dtype);
+    if (dtype == SDDMM_BF16 && K % 8) return fail(c, SDDMM_ERR_INVALID, "bf16 operands need K %% 8 == 0 (got %d)", K);
+    if ((M > 0 && !A) || (N > 0 && !B)) return fail(c, SDDMM_ERR_NULL, "A or B is NULL");
+    release_dense(c);
+    const size_t es = elem_size(dtype);
+    const size_t a_bytes = (size_t)M * K * es, b_bytes = (size_t)N * K * es;
+    if (on_device) {
+        if (((uintptr_t)A | (uintptr_t)B) & 15) return fail(c, SDDMM_ERR_INVALID, "device A/B must be 16-byte aligned");
+        c->dA = const_cast<void *>(A);
+        c->dB = const_cast<void *>(B);
+        c->own_dense = false;
+    } else {
+        c->own_dense = true;
+        ALLOC_TRY(c, c->dA, a_bytes);
+        ALLOC_TRY(c, c->dB, b_bytes);
+        if (a_bytes) HIP_TRY(c, hipMemcpyAsync(c->dA, A, a_bytes, hipMemcpyHostToDevice, c->stream));
+        if (b_bytes) HIP_TRY(c, hipMemcpyAsync(c->dB, B, b_bytes, hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipStreamSynchronize(c->stream));
+    }
+    c->M = M; c->N = N; c->K = K; c->dtype = dtype;
+    c->have_dense = true;
+    c->planned = false;
+    return SDDMM_OK;
+}
+
+int sddmm_set_dense(sddmm_ctx *c, int M, int N, int K, const void *A, const void *B, int dtype) {
+    return set_dense_common(c, M, N, K, A, B, dtype, false);
+}
+int sddmm_set_dense_device(sddmm_ctx *c, int M, int N, int K, const void *dA, const void *dB, int dtype) {
+    return set_dense_common(c, M, N, K, dA, dB, dtype, true);
+}
+
+int sddmm_set_csr(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *rowptr, const int32_t *col,
+                  const float *sval) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_dims(c, M, N, nnz);
+    if (rc) return rc;
+    if (!rowptr || (nnz > 0 && (!col || !sval))) return fail(c, SDDMM_ERR_NULL, "rowptr, col or values is NULL");
+    release_sparse(c);
+    c->own_sparse = c->own_rowptr = true;
+    ALLOC_TRY(c, c->d_rowptr, (size_t)(M + 1) * sizeof(int32_t));
+    ALLOC_TRY(c, c->d_col, (size_t)nnz * sizeof(int32_t));
+    ALLOC_TRY(c, c->d_sval, (size_t)nnz * sizeof(float));
+    ALLOC_TRY(c, c->dP, (size_t)nnz * sizeof(float));
+    HIP_TRY(c, hipMemcpyAsync(c->d_rowptr, rowptr, (size_t)(M + 1) * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+    if (nnz) {
+        HIP_TRY(c, hipMemcpyAsync(c->d_col, col, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipMemcpyAsync(c->d_sval, sval, (size_t)nnz * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipMemsetAsync(c->dP, 0, (size_t)nnz * sizeof(float), c->stream));
+    }
+    c->sM = M; c->sN = N; c->nnz = nnz;
+    rc = validate_csr(c);
+    if (rc) { release_sparse(c); return rc; }
+    c->have_sparse = c->have_rowptr = true;
+    return SDDMM_OK;
+}
+
+int sddmm_set_csr_device(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *d_rowptr, const int32_t *d_col,
+                         const float *d_sval) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_dims(c, M, N, nnz);
+    if (rc) return rc;
+    if (!d_rowptr || (nnz > 0 && (!d_col || !d_sval))) return fail(c, SDDMM_ERR_NULL, "rowptr, col or values is NULL");
+    release_sparse(c);
+    c->own_sparse = c->own_rowptr = false;
+    c->d_rowptr = const_cast<int32_t *>(d_rowptr);
+    c->d_col = const_cast<int32_t *>(d_col);
+    c->d_sval = const_cast<float *>(d_sval);
+    ALLOC_TRY(c, c->dP, (size_t)nnz * sizeof(float));
+    if (nnz) HIP_TRY(c, hipMemsetAsync(c->dP, 0, (size_t)nnz * sizeof(float), c->stream));
+    c->sM = M; c->sN = N; c->nnz = nnz;
+    rc = validate_csr(c);
+    if (rc) { release_sparse(c); return rc; }
+    c->have_sparse = c->have_rowptr = true;
+    return SDDMM_OK;
+}
+
+int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, const int32_t *col,
+                  const float *sval) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_dims(c, M, N, nnz);
+    if (rc) return rc;
+    if (nnz > 0 && (!row || !col || !sval)) return fail(c, SDDMM_ERR_NULL, "row, col or values is NULL");
+    release_sparse(c);
+    c->own_sparse = c->own_rowptr = c->own_rowidx = true;
+    c->from_coo = true;
+    ALLOC_TRY(c, c->d_rowidx, (size_t)nnz * sizeof(int32_t));
+    ALLOC_TRY(c, c->d_col, (size_t)nnz * sizeof(int32_t));
+    ALLOC_TRY(c, c->d_sval, (size_t)nnz * sizeof(float));
+    ALLOC_TRY(c, c->dP, (size_t)nnz * sizeof(float));
+    ALLOC_TRY(c, c->d_rowptr, (size_t)(M + 1) * sizeof(int32_t));
+    c->sM = M; c->sN = N; c->nnz = nnz;
+    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+    if (nnz) {
+        HIP_TRY(c, hipMemcpyAsync(c->d_rowidx, row, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipMemcpyAsync(c->d_col, col, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipMemcpyAsync(c->d_sval, sval, (size_t)nnz * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        HIP_TRY(c, hipMemsetAsync(c->dP, 0, (size_t)nnz * sizeof(float), c->stream));
+        const int g = grid_capped(nnz, 256);
+        hipLaunchKernelGGL(k_check_index, dim3(g), dim3(256), 0, c->stream, c->d_rowidx, nnz, M, c->d_pc);
+        hipLaunchKernelGGL(k_check_index, dim3(g), dim3(256), 0, c->stream, c->d_col, nnz, N, c->d_pc);
+        hipLaunchKernelGGL(k_check_coo_sorted, dim3(g), dim3(256), 0, c->stream, c->d_rowidx, nnz, c->d_pc);
+        HIP_TRY(c, hipGetLastError());
+    }
+    rc = fetch_counters(c);
+    if (rc) { release_sparse(c); return rc; }
+    if (c->pc.bad_pattern) {
+        release_sparse(c);
+        return fail(c, SDDMM_ERR_PATTERN, "COO row or column index out of range");
+    }
+    const bool sorted = c->pc.coo_unsorted == 0;
+    if (sorted) {
+        hipLaunchKernelGGL(k_rowptr_from_sorted_coo, dim3(grid_for(nnz + 1, 256)), dim3(256), 0, c->stream,
+                           c->d_rowidx, nnz, M, c->d_rowptr);
+        HIP_TRY(c, hipGetLastError());
+        HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+        if (M > 0)
+            hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(M, 256)), dim3(256), 0, c->stream, c->d_rowptr, M, nnz,
+                               c->d_pc);
+        HIP_TRY(c, hipGetLastError());
+        rc = fetch_counters(c);
+        if (rc) { release_sparse(c); return rc; }
+        if (c->pc.bad_pattern) {
+            release_sparse(c);
+            return fail(c, SDDMM_ERR_HIP, "internal: row pointer built from COO is inconsistent");
+        }
+        c->have_rowptr = true;
+    } else {
+        // row statistics are not available without a row pointer; count distinct rows as unknown
+        c->have_rowptr = false;
+        c->pc.rows_nonempty = 0;
+    }
+    c->have_sparse = true;
+    return SDDMM_OK;
+}
+
+int sddmm_update_values(sddmm_ctx *c, const float *sval) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    if (!c->have_sparse) return fail(c, SDDMM_ERR_STATE, "no sparse operand set");
+    if (!c->own_sparse) return fail(c, SDDMM_ERR_STATE, "values are caller-owned device memory");
+    if (c->nnz > 0 && !sval) return fail(c, SDDMM_ERR_NULL, "values is NULL");
+    if (c->nnz) HIP_TRY(c, hipMemcpyAsync(c->d_sval, sval, (size_t)c->nnz * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+static int check_ready(sddmm_ctx *c) {
+    if (!c->have_dense || !c->have_sparse) return fail(c, SDDMM_ERR_STATE, "set dense and sparse operands first");
+    if (c->sM > c->M || c->sN > c->N)
+        return fail(c, SDDMM_ERR_INVALID, "S is %dx%d but A has %d rows and B has %d rows", c->sM, c->sN, c->M, c->N);
+    return SDDMM_OK;
+}
+
+int sddmm_plan(sddmm_ctx *c, int strategy) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
+    rc = do_plan(c, strategy);
+    if (rc) return rc;
+    HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
+    HIP_TRY(c, hipEventSynchronize(c->ev1));
+    float ms = 0.f;
+    HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    c->stats = sddmm_stats{};
+    c->stats.plan_ms = ms;
+    fill_model(c);
+    return SDDMM_OK;
+}
+
+int sddmm_launch(sddmm_ctx *c) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    if (!c->planned) {
+        rc = sddmm_plan(c, SDDMM_AUTO);
+        if (rc) return rc;
+    }
+    return enqueue_run(c);
+}
+
+int sddmm_synchronize(sddmm_ctx *c) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+int sddmm_run(sddmm_ctx *c) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    if (!c->planned) {
+        rc = sddmm_plan(c, SDDMM_AUTO);
+        if (rc) return rc;
+    }
+    HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
+    rc = enqueue_run(c);
+    if (rc) return rc;
+    HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
+    HIP_TRY(c, hipEventSynchronize(c->ev1));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    float ms = 0.f;
+    HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    c->stats.run_ms = ms;
+    c->stats.kernels_launched = c->nnz ? 1 : 0;
+    return SDDMM_OK;
+}
+
+int sddmm_time_runs(sddmm_ctx *c, int warmup, int reps, int include_plan, float *ms_each) {
+    if (!c) return SDDMM_ERR_NULL;
+    if (reps < 0 || warmup < 0) return fail(c, SDDMM_ERR_INVALID, "negative repetition count");
+    if (reps > 0 && !ms_each) return fail(c, SDDMM_ERR_NULL, "ms_each is NULL");
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    if (!c->planned) {
+        rc = sddmm_plan(c, SDDMM_AUTO);
+        if (rc) return rc;
+    }
+    const int requested = c->requested;
+    for (int i = 0; i < warmup + reps; ++i) {
+        HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
+        if (include_plan) {
+            rc = do_plan(c, requested);
+            if (rc) return rc;
+        }
+        rc = enqueue_run(c);
+        if (rc) return rc;
+        HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
+        HIP_TRY(c, hipEventSynchronize(c->ev1));
+        if (i >= warmup) HIP_TRY(c, hipEventElapsedTime(&ms_each[i - warmup], c->ev0, c->ev1));
+    }
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+int sddmm_get_values(sddmm_ctx *c, float *P_values) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    if (!c->have_sparse) return fail(c, SDDMM_ERR_STATE, "no sparse operand set");
+    if (c->nnz > 0 && !P_values) return fail(c, SDDMM_ERR_NULL, "P_values is NULL");
+    if (c->nnz) HIP_TRY(c, hipMemcpyAsync(P_values, c->dP, (size_t)c->nnz * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+int sddmm_get_values_device(sddmm_ctx *c, const float **dP) {
+    if (!c || !dP) return SDDMM_ERR_NULL;
+    if (!c->have_sparse) return fail(c, SDDMM_ERR_STATE, "no sparse operand set");
+    *dP = c->dP;
+    return SDDMM_OK;
+}
+
+int sddmm_last_stats(const sddmm_ctx *c, sddmm_stats *out) {
+    if (!c || !out) return SDDMM_ERR_NULL;
+    *out = c->stats;
+    return SDDMM_OK;
+}
+
+// Smallest feasible maximum load by bisection, then a greedy left-to-right fill
+// with that load: the contract of CSR<T>::_dispatch (src/matrices/CSR.hpp:196-264).
+int sddmm_partition_rows(int M, const int32_t *rowptr, int parts, int stride, int32_t *start_idx) {
+    if (!rowptr || !start_idx) return SDDMM_ERR_NULL;
+    if (M <= 0 || parts <= 0 || stride <= 0 || M % stride) return SDDMM_ERR_INVALID;
+    const int64_t groups = M / stride;
+    auto load = [&](int64_t g) { return (int64_t)rowptr[(g + 1) * stride] - (int64_t)rowptr[g * stride]; };
+    int64_t heaviest = 0;
+    for (int64_t g = 0; g < groups; ++g) heaviest = std::max(heaviest, load(g));
+    auto parts_needed = [&](int64_t cap) {
+        int64_t used = 1, acc = 0;
+        for (int64_t g = 0; g < groups; ++g) {
+            acc += load(g);
+            if (acc > cap) { ++used; acc = load(g); }
+        }
+        return used;
+    };
+    int64_t lo = std::max<int64_t>(1, heaviest), hi = std::max<int64_t>(lo, rowptr[M]);
+    int64_t cap = 0;                       // stays 0 when even cap == nnz needs too many parts
+    if (parts_needed(hi) <= parts) {
+        while (lo < hi) {
+            const int64_t mid = lo + (hi - lo) / 2;
+            if (parts_needed(mid) <= parts) hi = mid; else lo = mid + 1;
+        }
+        cap = lo;
+    }
+    int w = 0;
+    int64_t acc = 0;
+    start_idx[w++] = 0;
+    for (int64_t g = 0; g < groups; ++g) {
+        acc += load(g);
+        if (acc > cap) {
+            if (w > parts) return SDDMM_ERR_INVALID;
+            start_idx[w++] = (int32_t)(g * stride);
+            acc = load(g);
+        }
+    }
+    while (w <= parts) start_idx[w++] = M;
+    return SDDMM_OK;
+}
+
+}  // extern "C"

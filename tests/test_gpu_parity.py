@@ -1,0 +1,297 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle.  All GPU.
+
+Bar: pattern and entry order bit-exact (P is returned in the caller's order by
+construction, checked through per-entry comparison); fp32 values within
+1e-5 * max(|ref|, 0.25 * |S| sum_k |a_k b_k|) of the oracle's fp32 k-ascending
+result (the floor covers entries whose terms cancel: both summation orders are
+equally accurate there and the pure relative error is unbounded); the EXACT
+strategy must be bit-identical to the oracle; bf16 inputs within 1e-2 on the
+same scale, the oracle consuming the bf16-rounded inputs.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from dphpc_amd import capi, workloads as W
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.EXACT]
+
+
+def _say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def run_csr(make, rowptr, col, sval, A, B, N, strategy, dtype=capi.F32):
+    e = make()
+    try:
+        e.set_dense(A, B, dtype)
+        e.set_csr(len(rowptr) - 1, N, rowptr, col, sval)
+        e.plan(strategy)
+        e.run()
+        return e.values(), e.stats()
+    finally:
+        e.close()
+
+
+def assert_parity(got, rowptr, col, sval, A, B, rtol=1e-5, exact=False, what=""):
+    ref = O.sddmm_csr(rowptr, col, sval, A, B, threads=0)
+    if exact:
+        bad = np.nonzero(got.view(np.uint32) != ref.view(np.uint32))[0]
+        assert len(bad) == 0, "%s: %d entries differ bitwise, first %d: %r vs %r" % (
+            what, len(bad), bad[0], got[bad[0]], ref[bad[0]])
+        return
+    _, mag = O.sddmm_csr_f64(rowptr, col, sval, A, B)
+    ok, worst, i = O.check_values(got, ref, mag=mag, rtol=rtol)
+    assert ok, "%s: entry %d got %r ref %r (%.2f x tolerance)" % (what, i, got[i], ref[i], worst)
+
+
+# ---- the reference's hand-checkable cases (tests/matrix_test.cc:124-182) -------
+KATS = {
+    "sddmm_coo1": ([[1, 2], [3, 4]], [[-1, 2], [-3, 4]], [(0, 0, 1), (0, 1, 1), (1, 0, 1), (1, 1, 1)], 2, 2, [3, 5, 5, 7]),
+    "sddmm_coo2": ([[1, 2, 3], [4, 5, 6]], [[-1, -3, 5], [2, 4, -6]], [(0, 0, 1), (1, 0, 1), (1, 1, 1)], 2, 2, [8, 11, -8]),
+    "sddmm_coo3": ([[1, 2, 3], [4, 5, 6]], [[-1, -3, 5]], [(0, 0, 1), (1, 0, -1)], 2, 1, [8, -11]),
+    "sddmm_coo4": ([[1, 2], [3, 4], [5, 6]], [[-1, -3], [2, 2], [3, 1]], [(0, 0, 1), (1, 0, -1), (2, 0, 1), (2, 2, 1)], 3, 3, [-7, 15, -23, 21]),
+    "dummy": ([[1, 1], [1, 1]], [[1, 1], [1, 1]], [(0, 0, 1), (0, 1, 1), (1, 0, 1), (1, 1, 1)], 2, 2, [2, 2, 2, 2]),
+}
+
+
+@pytest.mark.parametrize("name", list(KATS))
+@pytest.mark.parametrize("strategy", FP32_STRATEGIES)
+def test_reference_kats_csr_and_coo(engine_factory, name, strategy):
+    A, B, trip, M, N, exp = KATS[name]
+    A, B = np.array(A, f32), np.array(B, f32)
+    r = np.array([t[0] for t in trip], np.int32)
+    c = np.array([t[1] for t in trip], np.int32)
+    v = np.array([t[2] for t in trip], f32)
+    _say("KAT", name, capi.STRATEGY_NAMES[strategy])
+    rowptr, col, val = O.csr_from_triplets(M, r, c, v)
+    got, _ = run_csr(engine_factory, rowptr, col, val, A, B, N, strategy)
+    np.testing.assert_array_equal(got, np.array(exp, f32))       # small integers: exact in every order
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_coo(M, N, r, c, v)
+    e.plan(strategy)
+    e.run()
+    np.testing.assert_array_equal(e.values(), np.array(exp, f32))
+    e.close()
+
+
+def _random_case(rng, M, N, K, density, lo=-1.0):
+    mask = rng.random((M, N)) < density
+    r, c = np.nonzero(mask)
+    v = rng.uniform(lo, 1.0, len(r)).astype(f32)
+    A = rng.uniform(lo, 1.0, (M, K)).astype(f32)
+    B = rng.uniform(lo, 1.0, (N, K)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    return rowptr, col, val, A, B
+
+
+# the reference's randomized cross-checks (tests/matrix_test.cc:184-246), seeded here
+RANDOM_CASES = [(500, 500, 32, 0.3), (250, 250, 32, 0.7), (10000, 10000, 32, 0.001)]
+
+
+@pytest.mark.parametrize("case", RANDOM_CASES)
+@pytest.mark.parametrize("strategy", FP32_STRATEGIES)
+def test_random_matrices_like_the_reference_tests(engine_factory, case, strategy):
+    M, N, K, d = case
+    rng = np.random.default_rng(M + int(d * 1000))
+    rowptr, col, val, A, B = _random_case(rng, M, N, K, d)
+    _say("random", case, capi.STRATEGY_NAMES[strategy], "nnz", len(col))
+    got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, strategy)
+    assert st.nnz == len(col)
+    assert_parity(got, rowptr, col, val, A, B, exact=(strategy == capi.EXACT), what=str(case))
+
+
+# every K from 1 up, powers of two, multiples of 4 that are not powers of two,
+# odd K (scalar pieces) and K beyond one piece per lane
+KS = [1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 31, 32, 33, 48, 64, 96, 100, 128, 160, 256, 260, 300, 512, 1024]
+
+
+@pytest.mark.parametrize("K", KS)
+def test_any_k(engine_factory, K):
+    rng = np.random.default_rng(K)
+    rowptr, col, val, A, B = _random_case(rng, 150, 130, K, 0.25)
+    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.EXACT):
+        _say("K", K, capi.STRATEGY_NAMES[strategy])
+        got, _ = run_csr(engine_factory, rowptr, col, val, A, B, 130, strategy)
+        assert_parity(got, rowptr, col, val, A, B, exact=(strategy == capi.EXACT), what="K=%d" % K)
+
+
+def test_strategies_agree_bitwise(engine_factory):
+    # same per-entry arithmetic in every gather kernel
+    rng = np.random.default_rng(77)
+    for K in (32, 64, 20, 7, 128):
+        rowptr, col, val, A, B = _random_case(rng, 400, 300, K, 0.2)
+        a, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.FLAT)
+        b, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.ROW_WAVE)
+        c, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.AUTO)
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+        np.testing.assert_array_equal(a.view(np.uint32), c.view(np.uint32))
+
+
+def test_edge_shapes(engine_factory):
+    rng = np.random.default_rng(5)
+    K = 32
+    A = rng.uniform(-1, 1, (70, K)).astype(f32)
+    B = rng.uniform(-1, 1, (90, K)).astype(f32)
+    cases = {}
+    # empty matrix
+    cases["empty"] = (np.zeros(71, np.int32), np.zeros(0, np.int32), np.zeros(0, f32))
+    # single entry in the last row / last column
+    rp = np.zeros(71, np.int32); rp[70] = 1
+    cases["last"] = (rp, np.array([89], np.int32), np.array([2.0], f32))
+    # mostly empty rows, one full row, ragged lengths 0..69
+    lens = np.arange(70) % 7 == 0
+    lens = np.where(lens, np.arange(70), 0); lens[33] = 90
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(90, l, replace=False)) for l in lens]).astype(np.int32)
+    cases["ragged"] = (rp, col, rng.uniform(-1, 1, len(col)).astype(f32))
+    # explicit zeros in S stay stored and give exact zeros
+    rp = np.array([0] + [3] * 70, np.int32)
+    cases["zeros"] = (rp, np.array([1, 5, 9], np.int32), np.array([0.0, 1.0, -0.0], f32))
+    for name, (rowptr, col, val) in cases.items():
+        for strategy in FP32_STRATEGIES:
+            _say("edge", name, capi.STRATEGY_NAMES[strategy])
+            got, st = run_csr(engine_factory, rowptr, col, val, A, B, 90, strategy)
+            assert got.shape == (len(col),)
+            if len(col):
+                assert_parity(got, rowptr, col, val, A, B, exact=(strategy == capi.EXACT), what=name)
+    got, _ = run_csr(engine_factory, *cases["zeros"], A, B, 90, capi.AUTO)
+    assert got[0] == 0 and got[2] == 0
+
+
+def test_unsorted_columns_and_duplicates_keep_entry_order(engine_factory):
+    rng = np.random.default_rng(9)
+    K = 16
+    A = rng.uniform(-1, 1, (5, K)).astype(f32)
+    B = rng.uniform(-1, 1, (6, K)).astype(f32)
+    rowptr = np.array([0, 4, 4, 7, 8, 8], np.int32)
+    col = np.array([5, 0, 3, 0, 2, 2, 1, 4], np.int32)   # unsorted, duplicates
+    val = rng.uniform(-1, 1, 8).astype(f32)
+    for strategy in FP32_STRATEGIES:
+        got, _ = run_csr(engine_factory, rowptr, col, val, A, B, 6, strategy)
+        assert_parity(got, rowptr, col, val, A, B, exact=(strategy == capi.EXACT))
+    assert got[1] / val[1] == pytest.approx(got[3] / val[3], rel=1e-6)
+
+
+def test_coo_sorted_and_unsorted(engine_factory):
+    rng = np.random.default_rng(10)
+    rowptr, col, val, A, B = _random_case(rng, 300, 200, 32, 0.1)
+    rows = O.coo_rows_from_csr(rowptr)
+    ref = O.sddmm_coo(rows, col, val, A, B)
+    np.testing.assert_array_equal(ref, O.sddmm_csr(rowptr, col, val, A, B))
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    for strategy in FP32_STRATEGIES:
+        e = engine_factory()
+        e.set_dense(A, B)
+        e.set_coo(300, 200, rows, col, val)
+        e.plan(strategy)
+        e.run()
+        got = e.values()
+        e.close()
+        if strategy == capi.EXACT:
+            np.testing.assert_array_equal(got.view(np.uint32), ref.view(np.uint32))
+        else:
+            assert O.check_values(got, ref, mag=mag)[0]
+    # shuffled entries: output follows the caller's order
+    p = rng.permutation(len(col))
+    for strategy in (capi.AUTO, capi.FLAT, capi.EXACT):
+        e = engine_factory()
+        e.set_dense(A, B)
+        e.set_coo(300, 200, rows[p], col[p], val[p])
+        e.plan(strategy)
+        e.run()
+        got = e.values()
+        e.close()
+        assert O.check_values(got, ref[p], mag=mag[p])[0]
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_coo(300, 200, rows[p], col[p], val[p])
+    with pytest.raises(capi.SddmmError) as ei:
+        e.plan(capi.ROW_WAVE)
+    assert ei.value.code == capi.ERR_UNSUPPORTED
+    e.close()
+
+
+def test_error_paths_on_device(engine_factory):
+    e = engine_factory()
+    with pytest.raises(capi.SddmmError) as ei:
+        e.run()
+    assert ei.value.code == capi.ERR_STATE
+    A = np.ones((4, 8), f32); B = np.ones((5, 8), f32)
+    e.set_dense(A, B)
+    for rowptr, col, N in [
+        ([0, 2, 1, 3, 3], [0, 1, 2], 5),          # decreasing row pointer
+        ([1, 2, 3, 3, 3], [0, 1, 2], 5),          # does not start at 0
+        ([0, 1, 2, 3, 2], [0, 1, 2], 5),          # rowptr[M] != nnz
+        ([0, 1, 2, 3, 3], [0, 1, 5], 5),          # column out of range
+        ([0, 1, 2, 3, 3], [0, -1, 2], 5),
+    ]:
+        with pytest.raises(capi.SddmmError) as ei:
+            e.set_csr(4, N, np.array(rowptr, np.int32), np.array(col, np.int32), np.ones(len(col), f32))
+        assert ei.value.code == capi.ERR_PATTERN
+    with pytest.raises(capi.SddmmError) as ei:
+        e.set_coo(4, 5, np.array([0, 4], np.int32), np.array([0, 0], np.int32), np.ones(2, f32))
+    assert ei.value.code == capi.ERR_PATTERN
+    # S larger than the dense operands
+    e.set_csr(6, 5, np.zeros(7, np.int32), np.zeros(0, np.int32), np.zeros(0, f32))
+    with pytest.raises(capi.SddmmError) as ei:
+        e.plan(capi.AUTO)
+    assert ei.value.code == capi.ERR_INVALID
+    with pytest.raises(capi.SddmmError) as ei:
+        e.set_dense(np.ones((4, 12), np.uint16), np.ones((5, 12), np.uint16), capi.BF16)
+    assert ei.value.code == capi.ERR_INVALID
+    # a context stays usable after errors
+    e.set_dense(A, B)
+    e.set_csr(4, 5, np.array([0, 1, 1, 1, 2], np.int32), np.array([0, 4], np.int32), np.array([2, 3], f32))
+    e.run()
+    np.testing.assert_array_equal(e.values(), np.array([16, 24], f32))
+    e.close()
+
+
+def test_context_reuse_and_update_values(engine_factory):
+    # the harness reuses one competitor object for many runs and datasets
+    rng = np.random.default_rng(12)
+    e = engine_factory()
+    for M, N, K in [(100, 80, 32), (30, 200, 8), (100, 80, 32)]:
+        rowptr, col, val, A, B = _random_case(rng, M, N, K, 0.2)
+        e.set_dense(A, B)
+        e.set_csr(M, N, rowptr, col, val)
+        e.plan(capi.AUTO)
+        e.run()
+        assert_parity(e.values(), rowptr, col, val, A, B)
+        e.run()                                       # idempotent
+        assert_parity(e.values(), rowptr, col, val, A, B)
+        val2 = (val * f32(2)).astype(f32)
+        p1 = e.values()
+        e.update_values(val2)
+        e.run()
+        np.testing.assert_array_equal(e.values(), p1 * f32(2))   # linear in S, exactly for a factor 2
+    e.close()
+
+
+@pytest.mark.parametrize("name", ["small_uniform", "fem_banded", "power_law", "mixed_density"])
+def test_benchmark_shapes_scaled_down(engine_factory, name):
+    w = W.make(name, "small")
+    for strategy in FP32_STRATEGIES:
+        _say("shape", name, capi.STRATEGY_NAMES[strategy], "nnz", w.nnz)
+        got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, strategy)
+        assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, exact=(strategy == capi.EXACT), what=name)
+        assert st.flops == 2.0 * w.nnz * w.K
+        assert st.bytes_gathered == w.bytes_gathered()
+
+
+@pytest.mark.parametrize("K", [32, 128])
+def test_bf16_inputs_gather_path(engine_factory, K):
+    w = W.make("dense_tiles", "small", K=K)
+    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.EXACT):
+        _say("bf16", K, capi.STRATEGY_NAMES[strategy])
+        got, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A_bits, w.B_bits, w.N, strategy, capi.BF16)
+        # products of bf16 values are exact in fp32, accumulation is fp32: the fp32 bar applies
+        assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, rtol=1e-5, exact=(strategy == capi.EXACT), what="bf16")
