@@ -44,5 +44,21 @@ def build_library(verbose=False, extra_flags=()):
     return LIB_PATH
 
 
+PROBE_PATH = os.path.join(LIB_DIR, "copy_probe")
+
+
+def build_copy_probe(verbose=False):
+    """Stand-alone plain copy kernel used to calibrate rocprofv3's byte counters."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-o", PROBE_PATH, os.path.join(CSRC, "copy_probe.hip")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return PROBE_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_copy_probe(verbose=True))

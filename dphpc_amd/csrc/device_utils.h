@@ -17,8 +17,10 @@ constexpr int DPP_ROW_MIRROR = 0x140;      // lane i <-> 15-i inside each 16
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
+    // old = 0 with bound_ctrl lets the compiler fold the move into the consuming
+    // VALU instruction (v_add_f32_dpp); every pattern used here reads a valid lane
     int i = __builtin_bit_cast(int, v);
-    i = __builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false);
+    i = __builtin_amdgcn_update_dpp(0, i, CTRL, 0xF, 0xF, true);
     return __builtin_bit_cast(float, i);
 }
 

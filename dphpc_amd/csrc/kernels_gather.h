@@ -4,18 +4,20 @@
 // consecutive stored entries.  Lane l loads the column index / S value of entry
 // l of the chunk and finally stores its P value: plain coalesced 64-wide
 // accesses.  For the dot products the 64 lanes are cut into G = 64/LPN groups of
-// LPN lanes, LPN being the power of two >= K/ELEMS (capped at 64): at K=32 fp32 a
-// group is 8 lanes, each lane owning one 16-byte piece of a row, so a group reads
-// one contiguous 128-byte row of B.  In step t group g computes entry t*G+g, i.e.
-// a step covers G consecutive entries and a chunk of n entries needs ceil(n/G)
-// steps (a short chunk costs proportionally less).  Steps are issued in batches:
-// all gathers of a batch are in flight before the first FMA.  Lane (g*LPN+t)
-// keeps the group total of step t; one permute at the end brings entry l back to
-// lane l.
+// LPN lanes.  A row of K elements is KU units of 16 bytes; lane j of a group owns
+// units j, j+LPN, j+2*LPN, ... (UPL of them), so every load instruction has LPN
+// neighbouring lanes reading LPN*16 contiguous bytes of one row: at K=32 fp32,
+// LPN=8 and UPL=1, 8 lanes read one whole 128-byte B row (one cache line) per
+// instruction; at K=128, LPN=8 and UPL=4, four instructions read four lines.
+// In step t group g computes entry t*G+g, i.e. a step covers G
+// consecutive entries and a chunk of n entries needs ceil(n/G) steps (a short
+// chunk costs proportionally less).  Steps are issued in batches: all gathers of
+// a batch are in flight before the first FMA.  Lane (g*LPN+t) keeps the group
+// total of step t; one permute at the end brings entry l back to lane l.
 //
-// Per-entry arithmetic is the same everywhere (FMA chain over the lane's pieces
-// in k order, then the fixed tree of group_sum), so all strategies built from
-// these kernels return bit-identical values.
+// Per-entry arithmetic depends on K only (FMA chain over the lane's units in k
+// order, then the fixed tree of group_sum), so all strategies built from these
+// kernels return bit-identical values.
 #pragma once
 #include "device_utils.h"
 
@@ -24,63 +26,119 @@ namespace sddmm {
 constexpr int BLOCK = 256;                 // 4 wavefronts
 constexpr int WAVES_PER_BLOCK = BLOCK / WAVE;
 
-// Accumulates the dot products of up to 64 entries.
-//   U, LPN     unit type and lanes per entry
-//   WITH_ROWS  true: the A row differs per entry (r holds it per lane);
-//              false: `a` already holds this lane's piece of the one A row
-template <class U, int LPN, bool WITH_ROWS>
-struct ChunkSingle {
-    using T = typename U::T;
-    static constexpr int G = WAVE / LPN;
-    static constexpr int BIG = LPN < 8 ? LPN : 8;
-    static constexpr int SMALL = LPN < 2 ? LPN : 2;
+// Byte offset of a row: 32-bit when the whole operand is below 4 GiB (one VALU
+// multiply, scalar base + 32-bit vector offset addressing), 64-bit otherwise.
+template <bool WIDE> struct Off;
+template <> struct Off<false> { using T = uint32_t; };
+template <> struct Off<true> { using T = uint64_t; };
 
-    template <int NB>
-    static __device__ __forceinline__ void batch(int t0, const T *__restrict__ A, const T *__restrict__ B,
-                                                 int KU, int jj, bool lane_on, const T &a, int c, int r,
-                                                 int lane, float &out) {
-        const int g = lane / LPN, j = lane & (LPN - 1);
-        T bf[NB];
-        T af[WITH_ROWS ? NB : 1];
+template <class T, class O>
+__device__ __forceinline__ T load_at(const void *__restrict__ base, O byte_off) {
+    return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(base) + byte_off);
+}
+
+template <class O>
+__device__ __forceinline__ O shfl_off(O v, int src) {
+    if constexpr (sizeof(O) == 4) return (O)__shfl((int)v, src, WAVE);
+    else {
+        const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)v, src, WAVE);
+        const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)(v >> 32), src, WAVE);
+        return ((uint64_t)hi << 32) | lo;
+    }
+}
+
+// Dot products of up to 64 entries, one unit-set per lane.
+//   U, LPN, UPL  unit type, lanes per entry, units per lane (KU <= LPN*UPL)
+//   FULLK        KU == LPN*UPL: no lane is idle, no unit is masked
+//   WITH_ROWS    true: the A row differs per entry; false: `a` already holds the
+//                lane's units of the one A row
+//   WIDE         64-bit byte offsets
+template <class U, int LPN, int UPL, bool FULLK, bool WITH_ROWS, bool WIDE>
+struct Chunk {
+    using T = typename U::T;
+    using O = typename Off<WIDE>::T;
+    static constexpr int G = WAVE / LPN;
+    // gathers in flight per batch: about 8 x 16 bytes per lane (twice that with A)
+    static constexpr int NB_ = 8 / UPL < 1 ? 1 : 8 / UPL;
+    static constexpr int BIG = NB_ < LPN ? NB_ : LPN;
+    static constexpr int SMALL = 1;
+
+    struct Areg { T u[UPL]; };
+
+    static __device__ __forceinline__ bool unit_on(int j, int i, int KU) { return FULLK || (j + i * LPN) < KU; }
+
+    static __device__ __forceinline__ Areg load_a(const void *__restrict__ A, O row_off, int j, int KU) {
+        Areg a;
 #pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            const int src = ((t0 + u) * G + g) & (WAVE - 1);
-            const int cc = __shfl(c, src, WAVE);
-            bf[u] = B[(int64_t)cc * KU + jj];
-            if constexpr (WITH_ROWS) {
-                const int rr = __shfl(r, src, WAVE);
-                af[u] = A[(int64_t)rr * KU + jj];
+        for (int i = 0; i < UPL; ++i) {
+            const int u = unit_on(j, i, KU) ? j + i * LPN : 0;
+            a.u[i] = load_at<T, O>(A, row_off + (O)(u * (int)sizeof(T)));
+        }
+        return a;
+    }
+
+    template <int NB, class Hook>
+    static __device__ __forceinline__ void batch(int t0, const void *__restrict__ A, const void *__restrict__ B,
+                                                 int KU, const Areg &a, O boff, O aoff, int lane, float &out,
+                                                 Hook &&after_issue) {
+        const int g = lane / LPN, j = lane & (LPN - 1);
+        T bf[NB][UPL];
+        T af[WITH_ROWS ? NB : 1][UPL];
+#pragma unroll
+        for (int s = 0; s < NB; ++s) {
+            const int src = ((t0 + s) * G + g) & (WAVE - 1);
+            const O bo = shfl_off<O>(boff, src);
+            O ao = 0;
+            if constexpr (WITH_ROWS) ao = shfl_off<O>(aoff, src);
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                const int u = unit_on(j, i, KU) ? j + i * LPN : 0;
+                bf[s][i] = load_at<T, O>(B, bo + (O)(u * (int)sizeof(T)));
+                if constexpr (WITH_ROWS) af[s][i] = load_at<T, O>(A, ao + (O)(u * (int)sizeof(T)));
             }
         }
+        after_issue();
 #pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            float p;
-            if constexpr (WITH_ROWS) p = U::dot(af[u], bf[u], 0.f);
-            else p = U::dot(a, bf[u], 0.f);
-            p = group_sum<LPN>(lane_on ? p : 0.f);
-            if (j == t0 + u) out = p;
+        for (int s = 0; s < NB; ++s) {
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                float q;
+                if constexpr (WITH_ROWS) q = U::dot(af[s][i], bf[s][i], p);
+                else q = U::dot(a.u[i], bf[s][i], p);
+                p = unit_on(j, i, KU) ? q : p;
+            }
+            p = group_sum<LPN>(p);
+            if (j == t0 + s) out = p;
         }
     }
 
-    // c (and r) must be valid indices in every lane (0 for lanes past the end of
-    // the chunk); count = number of entries in the chunk (1..64).
-    static __device__ __forceinline__ float run(const T *__restrict__ A, const T *__restrict__ B, int KU,
-                                                const T &a, int c, int r, int count, int lane) {
-        const int j = lane & (LPN - 1);
-        const bool lane_on = j < KU;             // KU < LPN when K/ELEMS is not a power of two
-        const int jj = lane_on ? j : 0;
+    // boff / aoff: byte offset of this lane's entry's B row / A row (a valid row in
+    // every lane, row 0 past the end of the chunk); count = entries in the chunk.
+    // `prefetch` is called once, right after the first gathers have been issued:
+    // the place to start the index loads of the next chunk, so that they travel
+    // while this chunk computes (loads return in issue order, so anything issued
+    // before the gathers would have to land before them).
+    template <class Hook>
+    static __device__ __forceinline__ float run(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                const Areg &a, O boff, O aoff, int count, int lane,
+                                                Hook &&prefetch) {
         int steps = (count + G - 1) / G;
         steps = steps < LPN ? steps : LPN;
         float out = 0.f;
         int t0 = 0;
-        for (; t0 + BIG <= steps; t0 += BIG) batch<BIG>(t0, A, B, KU, jj, lane_on, a, c, r, lane, out);
-        for (; t0 < steps; t0 += SMALL) batch<SMALL>(t0, A, B, KU, jj, lane_on, a, c, r, lane, out);
+        bool fired = false;
+        auto once = [&]() { if (!fired) { prefetch(); fired = true; } };
+        for (; t0 + BIG <= steps; t0 += BIG) batch<BIG>(t0, A, B, KU, a, boff, aoff, lane, out, once);
+        if constexpr (BIG > 1)
+            for (; t0 < steps; t0 += SMALL) batch<SMALL>(t0, A, B, KU, a, boff, aoff, lane, out, once);
+        once();
         // entry l = t*G+g was kept by lane g*LPN+t
         return __shfl(out, (lane % G) * LPN + lane / G, WAVE);
     }
 };
 
-// K too long for one piece per lane (more than 64 units per row): one entry per
+// K too long for the register layout (more than 64 units per row): one entry per
 // step, all 64 lanes stride over the row.
 template <class U>
 __device__ __forceinline__ float chunk_long(const typename U::T *__restrict__ A,
@@ -100,43 +158,74 @@ __device__ __forceinline__ float chunk_long(const typename U::T *__restrict__ A,
     return out;
 }
 
+// Compile-time description of one (K, dtype) family.  LPN == 0 selects chunk_long.
+template <class U_, int LPN_, int UPL_, bool FULLK_, bool WIDE_>
+struct Layout {
+    using U = U_;
+    static constexpr int LPN = LPN_, UPL = UPL_;
+    static constexpr bool FULLK = FULLK_, WIDE = WIDE_, LONG = (LPN_ == 0);
+};
+
 // ---------------------------------------------------------------------------
 // FLAT: entries [0,nnz) in order, row index per entry read from rowidx (the COO
 // row array, or the expansion of rowptr built by the plan).  Perfectly balanced
-// whatever the row lengths are; A pieces are gathered per entry like B pieces
+// whatever the row lengths are; A units are gathered per entry like B units
 // (L1/L2 hits while the row does not change).
-template <class U, int LPN, bool SINGLE>
-__global__ __launch_bounds__(BLOCK) void k_flat(const typename U::T *__restrict__ A,
-                                                const typename U::T *__restrict__ B, int KU,
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_flat(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                 const int32_t *__restrict__ rowidx,
                                                 const int32_t *__restrict__ col,
                                                 const float *__restrict__ sval,
                                                 float *__restrict__ P, int64_t nnz,
                                                 int chunks_per_wave, int64_t nblocks) {
+    using U = typename L::U;
+    using T = typename U::T;
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int lane = lane_id();
     const int64_t wave = blk * WAVES_PER_BLOCK + wave_in_block();
     int64_t base = wave * (int64_t)chunks_per_wave * WAVE;
-    for (int ch = 0; ch < chunks_per_wave && base < nnz; ++ch, base += WAVE) {
+    if (base >= nnz) return;
+    int64_t stop = base + (int64_t)chunks_per_wave * WAVE;
+    stop = stop < nnz ? stop : nnz;
+    // Index loads are unconditional (clamped to the last entry of the range): lanes
+    // past the end then hold a valid row/column whose result is never stored, and
+    // the loads need no branch, which keeps the wait counts of the gathers exact.
+    const int64_t last = stop - 1;
+    const int64_t n0 = base + lane < last ? base + lane : last;
+    int c = col[n0], r = rowidx[n0];
+    float s = sval[n0];
+    for (; base < stop; base += WAVE) {
         const int64_t n = base + lane;
-        const bool valid = n < nnz;
-        const int c = valid ? col[n] : 0;
-        const int r = valid ? rowidx[n] : 0;
-        const float s = valid ? sval[n] : 0.f;
-        const int64_t left = nnz - base;
+        const bool valid = n < stop;
+        const int64_t left = stop - base;
         const int count = left < WAVE ? (int)left : WAVE;
+        int cn = 0, rn = 0;
+        float sn = 0.f;
+        auto prefetch = [&]() {
+            const int64_t pn = n + WAVE < last ? n + WAVE : last;
+            cn = col[pn]; rn = rowidx[pn]; sn = sval[pn];
+        };
         float res;
-        if constexpr (SINGLE) res = ChunkSingle<U, LPN, true>::run(A, B, KU, U::zero(), c, r, count, lane);
-        else res = chunk_long<U>(A, B, KU, c, r, count, lane);
+        if constexpr (L::LONG) {
+            prefetch();
+            res = chunk_long<U>((const T *)A, (const T *)B, KU, c, r, count, lane);
+        } else {
+            using C = Chunk<U, L::LPN, L::UPL, L::FULLK, true, L::WIDE>;
+            using O = typename C::O;
+            const O rb = (O)KU * (O)sizeof(T);
+            typename C::Areg none;
+            res = C::run(A, B, KU, none, (O)c * rb, (O)r * rb, count, lane, prefetch);
+        }
         if (valid) P[n] = res * s;
+        c = cn; r = rn; s = sn;
     }
 }
 
 // ---------------------------------------------------------------------------
 // ROW_WAVE: one wavefront per work item = a segment [start,end) of one row.
-// With items == nullptr item w is the whole row w.  The lane's piece of the A
-// row stays in a register for the whole segment; no row index is read.
+// With items == nullptr item w is the whole row w.  The lane's units of the A
+// row stay in registers for the whole segment; no row index is read.
 struct RowItem {
     int32_t row;
     int32_t start;
@@ -144,15 +233,16 @@ struct RowItem {
     int32_t pad;
 };
 
-template <class U, int LPN, bool SINGLE>
-__global__ __launch_bounds__(BLOCK) void k_row_wave(const typename U::T *__restrict__ A,
-                                                    const typename U::T *__restrict__ B, int KU,
-                                                    const int32_t *__restrict__ rowptr,
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_row_wave(const void *__restrict__ A, const void *__restrict__ B,
+                                                    int KU, const int32_t *__restrict__ rowptr,
                                                     const int32_t *__restrict__ col,
                                                     const float *__restrict__ sval,
                                                     float *__restrict__ P,
                                                     const RowItem *__restrict__ items,
                                                     int64_t n_items, int64_t nblocks) {
+    using U = typename L::U;
+    using T = typename U::T;
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
@@ -170,20 +260,40 @@ __global__ __launch_bounds__(BLOCK) void k_row_wave(const typename U::T *__restr
     end = __builtin_amdgcn_readfirstlane(end);
     if (start >= end) return;
     const int lane = lane_id();
-    const int j = lane & (LPN - 1);
-    typename U::T a = U::zero();
-    if constexpr (SINGLE) { if (j < KU) a = A[(int64_t)row * KU + j]; }
-    for (int base = start; base < end; base += WAVE) {
-        const int n = base + lane;
-        const bool valid = n < end;
-        const int c = valid ? col[n] : 0;
-        const float s = valid ? sval[n] : 0.f;
-        const int left = end - base;
-        const int count = left < WAVE ? left : WAVE;
-        float res;
-        if constexpr (SINGLE) res = ChunkSingle<U, LPN, false>::run(A, B, KU, a, c, 0, count, lane);
-        else res = chunk_long<U>(A, B, KU, c, row, count, lane);
-        if (valid) P[n] = res * s;
+    if constexpr (L::LONG) {
+        for (int base = start; base < end; base += WAVE) {
+            const int n = base + lane;
+            const bool valid = n < end;
+            const int c = valid ? col[n] : 0;
+            const float s = valid ? sval[n] : 0.f;
+            const int left = end - base;
+            const float res = chunk_long<U>((const T *)A, (const T *)B, KU, c, row, left < WAVE ? left : WAVE, lane);
+            if (valid) P[n] = res * s;
+        }
+    } else {
+        using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
+        using O = typename C::O;
+        const O rb = (O)KU * (O)sizeof(T);
+        const typename C::Areg a = C::load_a(A, (O)row * rb, lane & (L::LPN - 1), KU);
+        // unconditional, clamped index loads (see k_flat)
+        const int last = end - 1;
+        const int n0 = start + lane < last ? start + lane : last;
+        int c = col[n0];
+        float s = sval[n0];
+        for (int base = start; base < end; base += WAVE) {
+            const int n = base + lane;
+            const bool valid = n < end;
+            const int left = end - base;
+            int cn = 0;
+            float sn = 0.f;
+            auto prefetch = [&]() {
+                const int pn = n + WAVE < last ? n + WAVE : last;
+                cn = col[pn]; sn = sval[pn];
+            };
+            const float res = C::run(A, B, KU, a, (O)c * rb, (O)0, left < WAVE ? left : WAVE, lane, prefetch);
+            if (valid) P[n] = res * s;
+            c = cn; s = sn;
+        }
     }
 }
 

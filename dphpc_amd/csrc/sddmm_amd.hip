@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -116,83 +117,105 @@ int fetch_counters(sddmm_ctx *c) {
     return SDDMM_OK;
 }
 
-// power of two >= x, clamped to [1,64]
-int lanes_for(int units) {
+// ---- kernel dispatch over the (unit type, lanes per entry, units per lane) layouts ----
+struct Shape {
+    int unit;    // 0: fp32 x4, 1: fp32 x1, 2: bf16 x8
+    int KU;      // units per row
+    int LPN;     // lanes per entry (0: row too long for the register layout)
+    int UPL;     // units per lane
+    bool fullk;  // KU == LPN*UPL
+    bool wide;   // operands of 4 GiB or more: 64-bit byte offsets
+};
+
+int pow2ceil(int x) {
     int l = 1;
-    while (l < units && l < 64) l <<= 1;
+    while (l < x) l <<= 1;
     return l;
 }
 
-// ---- kernel dispatch over (unit type, lanes per entry) -----------------------
-struct Shape {
-    int unit;   // 0: fp32 x4, 1: fp32 x1, 2: bf16 x8
-    int KU;     // units per row
-    int LPN;    // lanes per entry
-    bool single;
-};
-
 Shape shape_of(const sddmm_ctx *c) {
     Shape s{};
-    if (c->dtype == SDDMM_BF16) { s.unit = 2; s.KU = c->K / 8; }
-    else if (c->K % 4 == 0) { s.unit = 0; s.KU = c->K / 4; }
-    else { s.unit = 1; s.KU = c->K; }
-    s.LPN = lanes_for(s.KU);
-    s.single = s.KU <= s.LPN;
+    size_t unit_bytes;
+    if (c->dtype == SDDMM_BF16) { s.unit = 2; s.KU = c->K / 8; unit_bytes = 16; }
+    else if (c->K % 4 == 0) { s.unit = 0; s.KU = c->K / 4; unit_bytes = 16; }
+    else { s.unit = 1; s.KU = c->K; unit_bytes = 4; }
+    if (s.unit == 1) {
+        // 4-byte units: 16 lanes cover 64 contiguous bytes
+        if (s.KU <= 4) { s.LPN = 4; s.UPL = 1; }
+        else if (s.KU <= 16) { s.LPN = 16; s.UPL = 1; }
+        else if (s.KU <= 64) { s.LPN = 16; s.UPL = 4; }
+        else if (s.KU <= 128) { s.LPN = 16; s.UPL = 8; }
+        else { s.LPN = 0; s.UPL = 0; }
+    } else {
+        // 16-byte units: 8 lanes cover one whole 128-byte cache line per load
+        // instruction (measured faster than 4 lanes x 64 bytes: half the lines per
+        // instruction for the same bytes)
+        if (s.KU <= 8) { s.LPN = pow2ceil(s.KU); s.UPL = 1; }
+        else if (s.KU <= 64) { s.LPN = 8; s.UPL = pow2ceil((s.KU + 7) / 8); }
+        else if (s.KU <= 128) { s.LPN = 16; s.UPL = 8; }
+        else { s.LPN = 0; s.UPL = 0; }
+    }
+    s.fullk = s.LPN > 0 && s.KU == s.LPN * s.UPL;
+    const size_t rows = (size_t)std::max(c->M, c->N);
+    s.wide = rows * (size_t)s.KU * unit_bytes >= ((size_t)1 << 32);
     return s;
 }
 
-template <class U, int LPN, bool SINGLE>
-void launch_flat_t(sddmm_ctx *c, int KU) {
+// Calls f(Layout<...>{}) for the layout matching s.
+template <class U, int LPN, int UPL, class F>
+void with_mask_width(const Shape &s, F &&f) {
+    if (s.wide) f(Layout<U, LPN, UPL, false, true>{});
+    else if (s.fullk && U::ELEMS > 1) f(Layout<U, LPN, UPL, true, false>{});
+    else f(Layout<U, LPN, UPL, false, false>{});
+}
+
+template <class U, class F>
+void with_layout16(const Shape &s, F &&f) {
+    if (s.LPN == 0) { f(Layout<U, 0, 1, false, true>{}); return; }
+    if (s.LPN == 1) with_mask_width<U, 1, 1>(s, f);
+    else if (s.LPN == 2) with_mask_width<U, 2, 1>(s, f);
+    else if (s.LPN == 4) with_mask_width<U, 4, 1>(s, f);
+    else if (s.LPN == 16) with_mask_width<U, 16, 8>(s, f);
+    else if (s.UPL == 1) with_mask_width<U, 8, 1>(s, f);
+    else if (s.UPL == 2) with_mask_width<U, 8, 2>(s, f);
+    else if (s.UPL == 4) with_mask_width<U, 8, 4>(s, f);
+    else with_mask_width<U, 8, 8>(s, f);
+}
+
+template <class F>
+void with_layout(const Shape &s, F &&f) {
+    if (s.unit == 0) with_layout16<UnitF32x4>(s, f);
+    else if (s.unit == 2) with_layout16<UnitBF16x8>(s, f);
+    else if (s.LPN == 0) f(Layout<UnitF32x1, 0, 1, false, true>{});
+    else if (s.LPN == 4) with_mask_width<UnitF32x1, 4, 1>(s, f);
+    else if (s.UPL == 1) with_mask_width<UnitF32x1, 16, 1>(s, f);
+    else if (s.UPL == 4) with_mask_width<UnitF32x1, 16, 4>(s, f);
+    else with_mask_width<UnitF32x1, 16, 8>(s, f);
+}
+
+void launch_flat(sddmm_ctx *c) {
+    const Shape s = shape_of(c);
     const int64_t chunks = (c->nnz + WAVE - 1) / WAVE;
-    int cpw = (int)std::min<int64_t>(8, std::max<int64_t>(1, chunks / (WAVES_PER_BLOCK * 4096)));
+    const int cpw = (int)std::min<int64_t>(8, std::max<int64_t>(1, chunks / (WAVES_PER_BLOCK * 4096)));
     const int64_t waves = (chunks + cpw - 1) / cpw;
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_flat<U, LPN, SINGLE>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
-                       (const typename U::T *)c->dA, (const typename U::T *)c->dB, KU, c->d_rowidx, c->d_col,
-                       c->d_sval, c->dP, c->nnz, cpw, nblocks);
+    with_layout(s, [&](auto L) {
+        using LT = decltype(L);
+        hipLaunchKernelGGL((k_flat<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowidx, c->d_col, c->d_sval, c->dP,
+                           c->nnz, cpw, nblocks);
+    });
 }
 
-template <class U, int LPN, bool SINGLE>
-void launch_row_wave_t(sddmm_ctx *c, int KU) {
-    const int64_t n_items = c->sM;
-    const int64_t nblocks = (n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_row_wave<U, LPN, SINGLE>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
-                       (const typename U::T *)c->dA, (const typename U::T *)c->dB, KU, c->d_rowptr, c->d_col,
-                       c->d_sval, c->dP, (const RowItem *)nullptr, n_items, nblocks);
-}
-
-enum class Kern { Flat, RowWave };
-
-template <class U, int LPN, bool SINGLE>
-void launch_kind(sddmm_ctx *c, Kern k, int KU) {
-    if (k == Kern::Flat) launch_flat_t<U, LPN, SINGLE>(c, KU);
-    else launch_row_wave_t<U, LPN, SINGLE>(c, KU);
-}
-
-template <class U, int LPN>
-void launch_single(sddmm_ctx *c, Kern k, const Shape &s) {
-    if (s.single) launch_kind<U, LPN, true>(c, k, s.KU);
-    else launch_kind<U, LPN, false>(c, k, s.KU);
-}
-
-template <class U>
-void launch_lpn(sddmm_ctx *c, Kern k, const Shape &s) {
-    switch (s.LPN) {
-        case 1: launch_single<U, 1>(c, k, s); break;
-        case 2: launch_single<U, 2>(c, k, s); break;
-        case 4: launch_single<U, 4>(c, k, s); break;
-        case 8: launch_single<U, 8>(c, k, s); break;
-        case 16: launch_single<U, 16>(c, k, s); break;
-        case 32: launch_single<U, 32>(c, k, s); break;
-        default: launch_single<U, 64>(c, k, s); break;
-    }
-}
-
-void launch_gather(sddmm_ctx *c, Kern k) {
+void launch_row_wave(sddmm_ctx *c, const RowItem *items, int64_t n_items) {
     const Shape s = shape_of(c);
-    if (s.unit == 0) launch_lpn<UnitF32x4>(c, k, s);
-    else if (s.unit == 1) launch_lpn<UnitF32x1>(c, k, s);
-    else launch_lpn<UnitBF16x8>(c, k, s);
+    const int64_t nblocks = (n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    with_layout(s, [&](auto L) {
+        using LT = decltype(L);
+        hipLaunchKernelGGL((k_row_wave<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
+                           items, n_items, nblocks);
+    });
 }
 
 int ensure_rowidx(sddmm_ctx *c) {
@@ -238,8 +261,8 @@ int check_dims(sddmm_ctx *c, int M, int N, int64_t nnz) {
 int enqueue_run(sddmm_ctx *c) {
     if (c->nnz == 0) return SDDMM_OK;
     switch (c->strategy) {
-        case SDDMM_FLAT: launch_gather(c, Kern::Flat); break;
-        case SDDMM_ROW_WAVE: launch_gather(c, Kern::RowWave); break;
+        case SDDMM_FLAT: launch_flat(c); break;
+        case SDDMM_ROW_WAVE: launch_row_wave(c, nullptr, c->sM); break;
         case SDDMM_EXACT:
             if (c->dtype == SDDMM_BF16)
                 hipLaunchKernelGGL(k_exact<true>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
@@ -261,11 +284,10 @@ int do_plan(sddmm_ctx *c, int strategy) {
         if (!csr_ok) resolved = SDDMM_FLAT;
         else {
             const double avg = c->sM ? (double)c->nnz / (double)c->sM : 0.0;
-            const Shape s = shape_of(c);
-            // whole-row waves pay off once a typical row fills the 64-entry step and
+            // whole-row waves pay off once a typical row fills a 64-entry chunk and
             // no single row dominates the run time
             const bool balanced = (double)c->pc.max_len <= 64.0 * std::max(avg, 1.0);
-            resolved = (avg >= 2.0 * (WAVE / s.LPN) && balanced) ? SDDMM_ROW_WAVE : SDDMM_FLAT;
+            resolved = (avg >= 32.0 && balanced) ? SDDMM_ROW_WAVE : SDDMM_FLAT;
         }
     }
     switch (resolved) {
