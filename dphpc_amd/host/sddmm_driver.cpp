@@ -1,0 +1,117 @@
+// Benchmark driver for the GPUAmd competitor: the role of the reference's
+// src/main.cpp + src/benchmark/benchmark.hpp for this one competitor family.
+//
+//   sddmm_driver [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx] [--no_csv_header]
+//
+// Prints one CSV line per run in the reference's 14-column schema
+// (src/main.cpp:356-358, src/benchmark/benchmark.hpp:95-98):
+//   competitor,dataset,mat_repr,M,N,K,NZ,total_ns,init_ns,comp_ns,cleanup_ns,
+//   correctness,num_thread_blocks,num_threads_per_block
+// init/cleanup/total are host wall-clock like the reference's; comp_ns is the
+// device time of run_* from HIP events recorded by the library on its launch
+// stream.  The correctness baseline is competitors[0] as in the reference
+// (benchmark.hpp:50-61); here that is GPU-AMD-Exact, the kernel that repeats the
+// CPU loop's operation order.
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <iostream>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "datasets.hpp"
+#include "gpu_amd.hpp"
+
+using Clock = std::chrono::high_resolution_clock;
+using sddmm_host::Dataset;
+
+struct Timing { long long total_ns, init_ns, comp_ns, cleanup_ns; };
+
+template <class F1, class F2, class F3>
+static Timing timed(Competitors::GPUAmd &c, F1 init, F2 run, F3 cleanup) {
+    const auto t0 = Clock::now();
+    init();
+    const auto t1 = Clock::now();
+    run();
+    const auto t2 = Clock::now();
+    cleanup();
+    const auto t3 = Clock::now();
+    auto ns = [](auto a, auto b) { return (long long)std::chrono::duration_cast<std::chrono::nanoseconds>(b - a).count(); };
+    Timing t{ns(t0, t3), ns(t0, t1), ns(t1, t2), ns(t2, t3)};
+    if (c.last_ok()) t.comp_ns = (long long)(c.last_stats().run_ms * 1e6);
+    return t;
+}
+
+static void bench_dataset(Dataset &d, std::vector<std::shared_ptr<Competitors::GPUAmd>> &comps, int num_runs) {
+    CSR<float> expected_csr(d.S_csr);
+    COO<float> expected_coo(d.S_coo);
+    bool have_expected = false;
+    const int K = (int)d.A.getCols();
+    for (auto &cp : comps) {
+        Competitors::GPUAmd &c = *cp;
+        for (int fmt = 0; fmt < 2; ++fmt) {
+            for (int run = 0; run < num_runs; ++run) {
+                Timing t;
+                bool correct;
+                if (fmt == 0) {
+                    CSR<float> P(d.S_csr);
+                    P.clearValues();
+                    t = timed(c, [&] { c.init_csr(d.A, d.B, d.S_csr, P); }, [&] { c.run_csr(d.A, d.B, d.S_csr, P); },
+                              [&] { c.cleanup_csr(d.A, d.B, d.S_csr, P); });
+                    if (!have_expected) { expected_csr = P; expected_coo = COO<float>(P); have_expected = c.last_ok(); }
+                    correct = c.last_ok() && P == expected_csr;
+                } else {
+                    COO<float> P(d.S_coo);
+                    P.clearValues();
+                    t = timed(c, [&] { c.init_coo(d.A, d.B, d.S_coo, P); }, [&] { c.run_coo(d.A, d.B, d.S_coo, P); },
+                              [&] { c.cleanup_coo(d.A, d.B, d.S_coo, P); });
+                    correct = c.last_ok() && P == expected_coo;
+                }
+                std::cout << c.name << "," << d.name << "," << (fmt == 0 ? "CSR" : "COO") << "," << d.S_coo.getRows() << ","
+                          << d.S_coo.getCols() << "," << K << "," << d.S_coo.getValues().size() << "," << t.total_ns << ","
+                          << t.init_ns << "," << t.comp_ns << "," << t.cleanup_ns << "," << correct << ","
+                          << c.get_num_thread_blocks() << "," << c.get_num_threads_per_block() << std::endl;
+            }
+        }
+    }
+}
+
+int main(int argc, char **argv) {
+    int K = 32, num_runs = 3;
+    double scale = 0.1;
+    bool header = true;
+    std::string only;
+    for (int i = 1; i < argc; ++i) {
+        const std::string a = argv[i];
+        auto next = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };
+        if (a == "--K" || a == "-k") K = std::atoi(next());
+        else if (a == "--num_runs") num_runs = std::atoi(next());
+        else if (a == "--scale") scale = std::atof(next());
+        else if (a == "--dataset" || a == "-d") only = next();
+        else if (a == "--no_csv_header") header = false;
+        else { std::fprintf(stderr, "usage: %s [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx] [--no_csv_header]\n", argv[0]); return 2; }
+    }
+    if (K < 1 || num_runs < 1 || scale <= 0) { std::fprintf(stderr, "bad arguments\n"); return 2; }
+    std::vector<std::shared_ptr<Competitors::GPUAmd>> comps;
+    for (int st : {SDDMM_EXACT, SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE}) comps.push_back(std::make_shared<Competitors::GPUAmd>(st));
+    if (header)
+        std::cout << "competitor,dataset,mat_repr,M,N,K,NZ,total_ns,init_ns,comp_ns,cleanup_ns,correctness,num_thread_blocks,num_threads_per_block" << std::endl;
+    auto want = [&](const char *n) { return only.empty() || only == n; };
+    auto dim = [&](int full, int mult) { return std::max(mult, (int)(full * scale) / mult * mult); };
+    const uint64_t seed = 0x5DD3300;
+    if (only.size() > 4 && only.substr(only.size() - 4) == ".mtx") {
+        Dataset d;
+        std::string err;
+        if (!sddmm_host::read_matrix_market(only, K, seed, d, err)) { std::fprintf(stderr, "%s: %s\n", only.c_str(), err.c_str()); return 1; }
+        bench_dataset(d, comps, num_runs);
+        return 0;
+    }
+    if (want("small_uniform")) { Dataset d = sddmm_host::uniform_random(656, 656, K, 0.044, seed + 1); d.name = "small_uniform"; bench_dataset(d, comps, num_runs); }
+    if (want("fem_banded")) { Dataset d = sddmm_host::fem_banded(dim(36000, 8), K, dim(3000, 8), 49.4, seed + 2); bench_dataset(d, comps, num_runs); }
+    if (want("power_law")) { Dataset d = sddmm_host::power_law(dim(2600000, 1), K, 13.85, 50000, seed + 3); bench_dataset(d, comps, num_runs); }
+    if (want("mixed_density")) { Dataset d = sddmm_host::mixed_density(dim(30000, 1), K, 0.10, 1385, 0.40, seed + 4); bench_dataset(d, comps, num_runs); }
+    if (want("dense_tiles")) { Dataset d = sddmm_host::dense_tiles(dim(4562, 16), dim(5761, 16), K, 0.094, seed + 5); bench_dataset(d, comps, num_runs); }
+    return 0;
+}
