@@ -11,8 +11,13 @@
 // device time of run_* from HIP events recorded by the library on its launch
 // stream.  The correctness baseline is competitors[0] as in the reference
 // (benchmark.hpp:50-61); here that is GPU-AMD-Exact, the kernel that repeats the
-// CPU loop's operation order.
+// CPU loop's operation order.  A run counts as correct when the pattern is
+// identical and every value is within 1e-5 * max(|expected|, 0.25 * mag) where
+// mag = |S| * sum_k |a_k b_k| is obtained from one more SDDMM on the absolute
+// values of the operands: with signed inputs some entries cancel almost to zero
+// and a purely relative test (the reference's, CSR.hpp:92-94) is meaningless there.
 #include <chrono>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -44,10 +49,39 @@ static Timing timed(Competitors::GPUAmd &c, F1 init, F2 run, F3 cleanup) {
     return t;
 }
 
+// |S| * sum_k |a_k * b_k| per stored entry, computed by the exact-order kernel
+static std::vector<float> magnitudes(Dataset &d) {
+    auto absd = [](Dense<float> &m) {
+        std::vector<float> flat(m.get_pointer(), m.get_pointer() + (size_t)m.getRows() * m.getCols());
+        for (auto &x : flat) x = std::fabs(x);
+        return Dense<float>(m.getRows(), m.getCols(), std::move(flat));
+    };
+    Dense<float> A = absd(d.A), B = absd(d.B);
+    CSR<float> S(d.S_csr);
+    for (auto &v : S.getValues()) v = std::fabs(v);
+    CSR<float> P(S);
+    P.clearValues();
+    Competitors::GPUAmd c(SDDMM_EXACT);
+    c.init_csr(A, B, S, P);
+    c.run_csr(A, B, S, P);
+    c.cleanup_csr(A, B, S, P);
+    return P.getValues();
+}
+
+static bool values_ok(const std::vector<float> &got, const std::vector<float> &exp, const std::vector<float> &mag) {
+    if (got.size() != exp.size() || got.size() != mag.size()) return false;
+    for (size_t i = 0; i < got.size(); ++i) {
+        const double scale = std::max(std::fabs((double)exp[i]), 0.25 * (double)mag[i]);
+        if (!(std::fabs((double)got[i] - (double)exp[i]) <= 1e-5 * scale)) return false;
+    }
+    return true;
+}
+
 static void bench_dataset(Dataset &d, std::vector<std::shared_ptr<Competitors::GPUAmd>> &comps, int num_runs) {
     CSR<float> expected_csr(d.S_csr);
     COO<float> expected_coo(d.S_coo);
     bool have_expected = false;
+    const std::vector<float> mag = magnitudes(d);
     const int K = (int)d.A.getCols();
     for (auto &cp : comps) {
         Competitors::GPUAmd &c = *cp;
@@ -61,13 +95,17 @@ static void bench_dataset(Dataset &d, std::vector<std::shared_ptr<Competitors::G
                     t = timed(c, [&] { c.init_csr(d.A, d.B, d.S_csr, P); }, [&] { c.run_csr(d.A, d.B, d.S_csr, P); },
                               [&] { c.cleanup_csr(d.A, d.B, d.S_csr, P); });
                     if (!have_expected) { expected_csr = P; expected_coo = COO<float>(P); have_expected = c.last_ok(); }
-                    correct = c.last_ok() && P == expected_csr;
+                    correct = c.last_ok() && P.getRowPositions() == expected_csr.getRowPositions() &&
+                              P.getColPositions() == expected_csr.getColPositions() &&
+                              values_ok(P.getValues(), expected_csr.getValues(), mag);
                 } else {
                     COO<float> P(d.S_coo);
                     P.clearValues();
                     t = timed(c, [&] { c.init_coo(d.A, d.B, d.S_coo, P); }, [&] { c.run_coo(d.A, d.B, d.S_coo, P); },
                               [&] { c.cleanup_coo(d.A, d.B, d.S_coo, P); });
-                    correct = c.last_ok() && P == expected_coo;
+                    correct = c.last_ok() && P.getRowPositions() == expected_coo.getRowPositions() &&
+                              P.getColPositions() == expected_coo.getColPositions() &&
+                              values_ok(P.getValues(), expected_coo.getValues(), mag);
                 }
                 std::cout << c.name << "," << d.name << "," << (fmt == 0 ? "CSR" : "COO") << "," << d.S_coo.getRows() << ","
                           << d.S_coo.getCols() << "," << K << "," << d.S_coo.getValues().size() << "," << t.total_ns << ","
