@@ -34,10 +34,10 @@ def sources():
     return [os.path.join(CSRC, "sddmm_amd.hip")]
 
 
-def build_library(verbose=False, extra_flags=()):
+def build_library(verbose=False, extra_flags=(), out=None):
     """(Re)build dphpc_amd/lib/libsddmm_amd.so; returns its path."""
     os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc()] + HIPCC_FLAGS + list(extra_flags) + ["-o", LIB_PATH] + sources()
+    cmd = [hipcc()] + HIPCC_FLAGS + list(extra_flags) + ["-o", out or LIB_PATH] + sources()
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

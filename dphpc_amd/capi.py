@@ -9,7 +9,8 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_PKG, "lib", "libsddmm_amd.so")
+# SDDMM_LIB selects another build of the same library (kernel experiments)
+_LIB_PATH = os.environ.get("SDDMM_LIB") or os.path.join(_PKG, "lib", "libsddmm_amd.so")
 
 AUTO, FLAT, ROW_WAVE, SHORT_ROWS, LDS_TILED, MFMA_TILE, EXACT = range(7)
 STRATEGY_NAMES = ["AUTO", "FLAT", "ROW_WAVE", "SHORT_ROWS", "LDS_TILED", "MFMA_TILE", "EXACT"]

@@ -59,6 +59,38 @@ inline int64_t xcd_grid(int64_t nblocks) {
     return ((nblocks + NUM_XCD - 1) / NUM_XCD) * NUM_XCD;
 }
 
+// Streamed operands (column indices, S values, row indices, P) are touched once
+// per run.  Marking them non-temporal (SDDMM_NT=1) was measured SLOWER on MI355X
+// (FEM-banded K=32: 119 us vs 86 us; power-law unchanged): repeated runs find the
+// index arrays in the last-level cache, and the hint gives that up.  Off by default.
+#ifndef SDDMM_NT
+#define SDDMM_NT 0
+#endif
+template <class T>
+__device__ __forceinline__ T ld_stream(const T *p) {
+#if SDDMM_NT
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+template <class T>
+__device__ __forceinline__ void st_stream(T *p, T v) {
+#if SDDMM_NT
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
+// One work item of the wave-per-segment kernel: entries [start,end) of one row.
+struct RowItem {
+    int32_t row;
+    int32_t start;
+    int32_t end;
+    int32_t pad;
+};
+
 // ---- units of the K dimension ----------------------------------------------
 // A "unit" is what one lane loads per step along K: 16 bytes where alignment
 // allows (4 fp32 or 8 bf16), one fp32 otherwise.  dot() extends an fp32

@@ -193,8 +193,8 @@ __global__ __launch_bounds__(BLOCK) void k_flat(const void *__restrict__ A, cons
     // the loads need no branch, which keeps the wait counts of the gathers exact.
     const int64_t last = stop - 1;
     const int64_t n0 = base + lane < last ? base + lane : last;
-    int c = col[n0], r = rowidx[n0];
-    float s = sval[n0];
+    int c = ld_stream(col + n0), r = ld_stream(rowidx + n0);
+    float s = ld_stream(sval + n0);
     for (; base < stop; base += WAVE) {
         const int64_t n = base + lane;
         const bool valid = n < stop;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(BLOCK) void k_flat(const void *__restrict__ A, cons
         float sn = 0.f;
         auto prefetch = [&]() {
             const int64_t pn = n + WAVE < last ? n + WAVE : last;
-            cn = col[pn]; rn = rowidx[pn]; sn = sval[pn];
+            cn = ld_stream(col + pn); rn = ld_stream(rowidx + pn); sn = ld_stream(sval + pn);
         };
         float res;
         if constexpr (L::LONG) {
@@ -217,22 +217,134 @@ __global__ __launch_bounds__(BLOCK) void k_flat(const void *__restrict__ A, cons
             typename C::Areg none;
             res = C::run(A, B, KU, none, (O)c * rb, (O)r * rb, count, lane, prefetch);
         }
-        if (valid) P[n] = res * s;
+        if (valid) st_stream(P + n, res * s);
         c = cn; r = rn; s = sn;
     }
 }
 
 // ---------------------------------------------------------------------------
-// ROW_WAVE: one wavefront per work item = a segment [start,end) of one row.
-// With items == nullptr item w is the whole row w.  The lane's units of the A
-// row stay in registers for the whole segment; no row index is read.
-struct RowItem {
-    int32_t row;
-    int32_t start;
-    int32_t end;
-    int32_t pad;
-};
+// Bodies shared by the stand-alone kernels and the fused AUTO kernel.
 
+// One wavefront, one work item = entries [start,end) of `row`.  The lane's units
+// of the A row stay in registers for the whole segment; no row index is read.
+template <class L>
+__device__ __forceinline__ void row_segment_body(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                 float *__restrict__ P, int row, int start, int end, int lane) {
+    using U = typename L::U;
+    using T = typename U::T;
+    if (start >= end) return;
+    if constexpr (L::LONG) {
+        for (int base = start; base < end; base += WAVE) {
+            const int n = base + lane;
+            const bool valid = n < end;
+            const int c = valid ? ld_stream(col + n) : 0;
+            const float s = valid ? ld_stream(sval + n) : 0.f;
+            const int left = end - base;
+            const float res = chunk_long<U>((const T *)A, (const T *)B, KU, c, row, left < WAVE ? left : WAVE, lane);
+            if (valid) st_stream(P + n, res * s);
+        }
+    } else {
+        using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
+        using O = typename C::O;
+        const O rb = (O)KU * (O)sizeof(T);
+        const typename C::Areg a = C::load_a(A, (O)row * rb, lane & (L::LPN - 1), KU);
+        // Index loads are unconditional (clamped to the last entry of the range): lanes
+        // past the end then hold a valid column whose result is never stored, and the
+        // loads need no branch, which keeps the wait counts of the gathers exact.
+        const int last = end - 1;
+        const int n0 = start + lane < last ? start + lane : last;
+        int c = ld_stream(col + n0);
+        float s = ld_stream(sval + n0);
+        for (int base = start; base < end; base += WAVE) {
+            const int n = base + lane;
+            const bool valid = n < end;
+            const int left = end - base;
+            int cn = 0;
+            float sn = 0.f;
+            auto prefetch = [&]() {
+                const int pn = n + WAVE < last ? n + WAVE : last;
+                cn = ld_stream(col + pn); sn = ld_stream(sval + pn);
+            };
+            const float res = C::run(A, B, KU, a, (O)c * rb, (O)0, left < WAVE ? left : WAVE, lane, prefetch);
+            if (valid) st_stream(P + n, res * s);
+            c = cn; s = sn;
+        }
+    }
+}
+
+// One wavefront, `rpw` consecutive rows starting at r0 (rpw <= 64); only rows with
+// fewer than `ts` entries are computed (the others belong to the segment items).
+// The entries of the short rows are numbered consecutively across the rows, so
+// the lanes stay full whatever the individual lengths are; the row of an entry is
+// found by bisection over the wave's inclusive prefix sums (registers only), one
+// chunk ahead, so that the index loads of chunk i+1 travel while chunk i computes.
+template <class L>
+__device__ __forceinline__ void short_rows_body(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                const int32_t *__restrict__ rowptr,
+                                                const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                float *__restrict__ P, int M, int ts, int64_t r0, int rpw, int lane) {
+    using U = typename L::U;
+    using T = typename U::T;
+    int rs = 0, len = 0;
+    if (lane < rpw && r0 + lane < M) {
+        rs = rowptr[r0 + lane];
+        len = rowptr[r0 + lane + 1] - rs;
+        if (len >= ts) len = 0;
+    }
+    int incl = len;
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const int up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
+    }
+    const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, WAVE - 1, WAVE));
+    if (total == 0) return;
+    const int excl = incl - len;
+    // entry index and row of virtual entry v (clamped to the last one)
+    auto locate = [&](int v, int &n, int &row) {
+        v = v < total ? v : total - 1;
+        int lo = 0;
+#pragma unroll
+        for (int step = WAVE / 2; step > 0; step >>= 1) {
+            const int probe = __shfl(incl, lo + step - 1, WAVE);
+            if (probe <= v) lo += step;
+        }
+        n = __shfl(rs, lo, WAVE) + (v - __shfl(excl, lo, WAVE));
+        row = (int)r0 + lo;
+    };
+    int n, row;
+    locate(lane, n, row);
+    int c = ld_stream(col + n);
+    float s = ld_stream(sval + n);
+    for (int base = 0; base < total; base += WAVE) {
+        const bool valid = base + lane < total;
+        const int left = total - base;
+        const int count = left < WAVE ? left : WAVE;
+        int nn = n, rown = row, cn = 0;
+        float sn = 0.f;
+        auto prefetch = [&]() {
+            locate(base + WAVE + lane, nn, rown);
+            cn = ld_stream(col + nn); sn = ld_stream(sval + nn);
+        };
+        float res;
+        if constexpr (L::LONG) {
+            prefetch();
+            res = chunk_long<U>((const T *)A, (const T *)B, KU, c, row, count, lane);
+        } else {
+            using C = Chunk<U, L::LPN, L::UPL, L::FULLK, true, L::WIDE>;
+            using O = typename C::O;
+            const O rb = (O)KU * (O)sizeof(T);
+            typename C::Areg none;
+            res = C::run(A, B, KU, none, (O)c * rb, (O)row * rb, count, lane, prefetch);
+        }
+        if (valid) st_stream(P + n, res * s);
+        n = nn; row = rown; c = cn; s = sn;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// ROW_WAVE: one wavefront per work item.  With items == nullptr item w is the
+// whole row w.
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_row_wave(const void *__restrict__ A, const void *__restrict__ B,
                                                     int KU, const int32_t *__restrict__ rowptr,
@@ -241,8 +353,6 @@ __global__ __launch_bounds__(BLOCK) void k_row_wave(const void *__restrict__ A, 
                                                     float *__restrict__ P,
                                                     const RowItem *__restrict__ items,
                                                     int64_t n_items, int64_t nblocks) {
-    using U = typename L::U;
-    using T = typename U::T;
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
@@ -258,42 +368,58 @@ __global__ __launch_bounds__(BLOCK) void k_row_wave(const void *__restrict__ A, 
     row = __builtin_amdgcn_readfirstlane(row);
     start = __builtin_amdgcn_readfirstlane(start);
     end = __builtin_amdgcn_readfirstlane(end);
-    if (start >= end) return;
-    const int lane = lane_id();
-    if constexpr (L::LONG) {
-        for (int base = start; base < end; base += WAVE) {
-            const int n = base + lane;
-            const bool valid = n < end;
-            const int c = valid ? col[n] : 0;
-            const float s = valid ? sval[n] : 0.f;
-            const int left = end - base;
-            const float res = chunk_long<U>((const T *)A, (const T *)B, KU, c, row, left < WAVE ? left : WAVE, lane);
-            if (valid) P[n] = res * s;
-        }
+    row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
+}
+
+// ---------------------------------------------------------------------------
+// SHORT_ROWS as a strategy of its own: every row counts as short (ts = INT_MAX).
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_short_rows(const void *__restrict__ A, const void *__restrict__ B,
+                                                      int KU, const int32_t *__restrict__ rowptr,
+                                                      const int32_t *__restrict__ col,
+                                                      const float *__restrict__ sval,
+                                                      float *__restrict__ P, int M, int ts, int rpw,
+                                                      int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t r0 = (blk * WAVES_PER_BLOCK + wave_in_block()) * rpw;
+    if (r0 >= M) return;
+    short_rows_body<L>(A, B, KU, rowptr, col, sval, P, M, ts, r0, rpw, lane_id());
+}
+
+// ---------------------------------------------------------------------------
+// AUTO: one launch for both row classes.  Logical blocks [0, short_blocks) run the
+// many-rows-per-wave body over all rows (skipping the rows that have items), the
+// blocks after them run one segment item per wavefront.  The item blocks come
+// last in the XCD-contiguous order, after the short-row work of the same XCD.
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                const int32_t *__restrict__ rowptr,
+                                                const int32_t *__restrict__ col,
+                                                const float *__restrict__ sval, float *__restrict__ P, int M,
+                                                int ts, int rpw, int64_t short_blocks,
+                                                const RowItem *__restrict__ items, int64_t n_items,
+                                                int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    // interleave: the item blocks of a long-row-heavy matrix start early instead
+    // of forming a tail; block b is an item block when b*item_blocks/nblocks steps
+    const int64_t item_blocks = nblocks - short_blocks;
+    const int64_t items_before = blk * item_blocks / nblocks;
+    const bool is_item = ((blk + 1) * item_blocks / nblocks) != items_before;
+    if (is_item) {
+        const int64_t w = items_before * WAVES_PER_BLOCK + wave_in_block();
+        if (w >= n_items) return;
+        const RowItem it = items[w];
+        const int row = __builtin_amdgcn_readfirstlane(it.row);
+        const int start = __builtin_amdgcn_readfirstlane(it.start);
+        const int end = __builtin_amdgcn_readfirstlane(it.end);
+        row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
     } else {
-        using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
-        using O = typename C::O;
-        const O rb = (O)KU * (O)sizeof(T);
-        const typename C::Areg a = C::load_a(A, (O)row * rb, lane & (L::LPN - 1), KU);
-        // unconditional, clamped index loads (see k_flat)
-        const int last = end - 1;
-        const int n0 = start + lane < last ? start + lane : last;
-        int c = col[n0];
-        float s = sval[n0];
-        for (int base = start; base < end; base += WAVE) {
-            const int n = base + lane;
-            const bool valid = n < end;
-            const int left = end - base;
-            int cn = 0;
-            float sn = 0.f;
-            auto prefetch = [&]() {
-                const int pn = n + WAVE < last ? n + WAVE : last;
-                cn = col[pn]; sn = sval[pn];
-            };
-            const float res = C::run(A, B, KU, a, (O)c * rb, (O)0, left < WAVE ? left : WAVE, lane, prefetch);
-            if (valid) P[n] = res * s;
-            c = cn; s = sn;
-        }
+        const int64_t sb = blk - items_before;
+        const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
+        if (r0 >= M) return;
+        short_rows_body<L>(A, B, KU, rowptr, col, sval, P, M, ts, r0, rpw, lane_id());
     }
 }
 

@@ -110,3 +110,122 @@ __global__ __launch_bounds__(256) void k_rowptr_from_sorted_coo(const int32_t *_
 }
 
 }  // namespace sddmm
+
+// ===========================================================================
+// Row classifier of the AUTO strategy.
+//
+// A row is "short" when it has fewer than `ts` stored entries; short rows are
+// computed by k_short_rows straight from rowptr, 64 consecutive rows per
+// wavefront, and need no list.  Every other row becomes ceil(len/seg) work items
+// of the wave-per-segment kernel; the item list is built with an exclusive scan
+// of the per-row item counts (three kernels: block sums, scan of the block sums,
+// write).  Nothing here touches col/values: the cost is O(M).
+namespace sddmm {
+
+constexpr int SCAN_BLOCK = 256;
+constexpr int SCAN_ITEMS = 4;                       // rows per thread
+constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;  // rows per block
+
+__device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr, int64_t i, int M,
+                                                       int ts, int seg, unsigned int *len_out) {
+    if (i >= M) { *len_out = 0; return 0; }
+    const unsigned int len = (unsigned int)(rowptr[i + 1] - rowptr[i]);
+    *len_out = len;
+    return len >= (unsigned int)ts ? (len + seg - 1) / seg : 0u;
+}
+
+// block-wide exclusive scan of one value per thread (SCAN_BLOCK threads); returns
+// the exclusive prefix, *total receives the block sum
+__device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, unsigned int *total) {
+    __shared__ unsigned int wave_sums[SCAN_BLOCK / WAVE];
+    const int lane = lane_id(), wid = threadIdx.x >> 6;
+    unsigned int incl = v;
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const unsigned int up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
+    }
+    if (lane == WAVE - 1) wave_sums[wid] = incl;
+    __syncthreads();
+    unsigned int before = 0, all = 0;
+    for (int w = 0; w < SCAN_BLOCK / WAVE; ++w) {
+        const unsigned int s = wave_sums[w];
+        if (w < wid) before += s;
+        all += s;
+    }
+    __syncthreads();
+    *total = all;
+    return before + incl - v;
+}
+
+// pass 1: items per block of SCAN_TILE rows, plus the row statistics
+__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr, int M, int ts,
+                                                               int seg, unsigned int *__restrict__ block_sums,
+                                                               PlanCounters *pc) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    unsigned int items = 0;
+    unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        unsigned int len;
+        const unsigned int cnt = row_item_count(rowptr, base + q, M, ts, seg, &len);
+        items += cnt;
+        if (len == 0) continue;
+        if (cnt == 0) { ++r_short; n_short += len; }
+        else if (cnt == 1) { ++r_med; n_med += len; }
+        else { ++r_long; n_long += len; }
+    }
+    unsigned int total;
+    (void)block_exclusive_scan(items, &total);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+    r_short = wave_sum_u64(r_short); r_med = wave_sum_u64(r_med); r_long = wave_sum_u64(r_long);
+    n_short = wave_sum_u64(n_short); n_med = wave_sum_u64(n_med); n_long = wave_sum_u64(n_long);
+    if (lane_id() == 0) {
+        if (r_short) atomicAdd(&pc->rows_short, r_short);
+        if (r_med) atomicAdd(&pc->rows_medium, r_med);
+        if (r_long) atomicAdd(&pc->rows_long, r_long);
+        if (n_short) atomicAdd(&pc->nnz_short, n_short);
+        if (n_med) atomicAdd(&pc->nnz_medium, n_med);
+        if (n_long) atomicAdd(&pc->nnz_long, n_long);
+    }
+}
+
+// pass 2: exclusive scan of the block sums in place (one workgroup), total -> pc->n_items
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__restrict__ block_sums, int n,
+                                                                PlanCounters *pc) {
+    unsigned int carry = 0;
+    for (int base = 0; base < n; base += SCAN_BLOCK) {
+        const int i = base + (int)threadIdx.x;
+        const unsigned int v = i < n ? block_sums[i] : 0u;
+        unsigned int total;
+        const unsigned int ex = block_exclusive_scan(v, &total);
+        if (i < n) block_sums[i] = carry + ex;
+        carry += total;
+    }
+    if (threadIdx.x == 0) pc->n_items = carry;
+}
+
+// pass 3: write the items
+__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr, int M, int ts,
+                                                               int seg, const unsigned int *__restrict__ block_offsets,
+                                                               RowItem *__restrict__ items) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    unsigned int cnt[SCAN_ITEMS], mine = 0;
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        unsigned int len;
+        cnt[q] = row_item_count(rowptr, base + q, M, ts, seg, &len);
+        mine += cnt[q];
+    }
+    unsigned int total;
+    unsigned int at = block_offsets[blockIdx.x] + block_exclusive_scan(mine, &total);
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        if (cnt[q] == 0) continue;
+        const int32_t row = (int32_t)(base + q);
+        const int32_t s = rowptr[row], e = rowptr[row + 1];
+        for (unsigned int k = 0; k < cnt[q]; ++k) {
+            const int32_t a = s + (int32_t)k * seg;
+            const int32_t b = a + seg < e ? a + seg : e;
+            items[at++] = RowItem{row, a, b, 0};
+        }
+    }
+}
+
+}  // namespace sddmm

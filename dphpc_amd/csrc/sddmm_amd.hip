@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <climits>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -45,6 +46,15 @@ struct sddmm_ctx {
     PlanCounters *d_pc = nullptr;    // device counters
     PlanCounters pc{};               // host copy
     sddmm_stats stats{};
+    // AUTO: rows shorter than ts go to the many-rows-per-wave kernel, the others
+    // become wave-per-segment items of at most seg entries
+    int ts = 0, seg = 0, rpw = 64;
+    RowItem *d_items = nullptr;
+    int64_t n_items = 0, items_cap = 0;
+    unsigned int *d_block_sums = nullptr;
+    int64_t block_sums_cap = 0;
+    int64_t rows_short = 0;
+    int launches = 0;
 };
 
 namespace {
@@ -96,6 +106,9 @@ void release_sparse(sddmm_ctx *c) {
     if (c->own_rowptr) dfree(c->d_rowptr);
     if (c->own_rowidx) dfree(c->d_rowidx);
     dfree(c->dP);
+    dfree(c->d_items);
+    dfree(c->d_block_sums);
+    c->items_cap = c->block_sums_cap = c->n_items = 0;
     c->d_col = nullptr; c->d_sval = nullptr; c->d_rowptr = nullptr; c->d_rowidx = nullptr;
     c->own_sparse = c->own_rowptr = c->own_rowidx = false;
     c->have_sparse = c->have_rowptr = false;
@@ -218,6 +231,86 @@ void launch_row_wave(sddmm_ctx *c, const RowItem *items, int64_t n_items) {
     });
 }
 
+// rows per wavefront of the many-rows body: about 256 short entries per wave, so
+// that small matrices still produce enough waves to fill the chip
+int rows_per_wave(double avg_short_len) {
+    int rpw = 64;
+    while (rpw > 8 && rpw * std::max(avg_short_len, 1.0) > 384.0) rpw >>= 1;
+    return rpw;
+}
+
+void launch_short_rows(sddmm_ctx *c, int ts, int rpw) {
+    const Shape s = shape_of(c);
+    const int64_t waves = ((int64_t)c->sM + rpw - 1) / rpw;
+    const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    with_layout(s, [&](auto L) {
+        using LT = decltype(L);
+        hipLaunchKernelGGL((k_short_rows<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
+                           c->sM, ts, rpw, nblocks);
+    });
+}
+
+void launch_auto(sddmm_ctx *c) {
+    const Shape s = shape_of(c);
+    const int64_t waves = c->rows_short > 0 ? ((int64_t)c->sM + c->rpw - 1) / c->rpw : 0;
+    const int64_t short_blocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t nblocks = short_blocks + item_blocks;
+    with_layout(s, [&](auto L) {
+        using LT = decltype(L);
+        hipLaunchKernelGGL((k_auto<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
+                           c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
+    });
+}
+
+int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : fallback;
+}
+
+// Row classifier: statistics, then the item list of the wave-per-segment kernel.
+int classify_rows(sddmm_ctx *c) {
+    const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
+    if (nb > c->block_sums_cap) {
+        dfree(c->d_block_sums);
+        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
+        c->block_sums_cap = nb;
+    }
+    // keep what validation measured, clear what the classifier accumulates
+    PlanCounters fresh = c->pc;
+    fresh.rows_short = fresh.rows_medium = fresh.rows_long = 0;
+    fresh.nnz_short = fresh.nnz_medium = fresh.nnz_long = 0;
+    fresh.n_items = 0;
+    c->pc = fresh;
+    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
+    if (nb > 0) {
+        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, c->sM,
+                           c->ts, c->seg, c->d_block_sums, c->d_pc);
+        hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
+                           c->d_pc);
+        HIP_TRY(c, hipGetLastError());
+    }
+    int rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_items = (int64_t)c->pc.n_items;
+    c->rows_short = (int64_t)c->pc.rows_short;
+    c->rpw = env_int("SDDMM_RPW", rows_per_wave(c->rows_short ? (double)c->pc.nnz_short / (double)c->rows_short : 0.0));
+    c->rpw = std::min(64, std::max(1, c->rpw));
+    if (c->n_items > c->items_cap) {
+        dfree(c->d_items);
+        ALLOC_TRY(c, c->d_items, (size_t)c->n_items * sizeof(RowItem));
+        c->items_cap = c->n_items;
+    }
+    if (c->n_items > 0) {
+        hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, c->sM,
+                           c->ts, c->seg, c->d_block_sums, c->d_items);
+        HIP_TRY(c, hipGetLastError());
+    }
+    return SDDMM_OK;
+}
+
 int ensure_rowidx(sddmm_ctx *c) {
     if (c->d_rowidx) return SDDMM_OK;
     ALLOC_TRY(c, c->d_rowidx, (size_t)c->nnz * sizeof(int32_t));
@@ -259,10 +352,19 @@ int check_dims(sddmm_ctx *c, int M, int N, int64_t nnz) {
 }
 
 int enqueue_run(sddmm_ctx *c) {
+    c->launches = 0;
     if (c->nnz == 0) return SDDMM_OK;
+    c->launches = 1;
     switch (c->strategy) {
+        case SDDMM_AUTO:
+            if (c->rows_short == 0 && c->n_items == 0) { c->launches = 0; break; }
+            launch_auto(c);
+            break;
         case SDDMM_FLAT: launch_flat(c); break;
         case SDDMM_ROW_WAVE: launch_row_wave(c, nullptr, c->sM); break;
+        case SDDMM_SHORT_ROWS:
+            launch_short_rows(c, INT32_MAX, rows_per_wave(c->sM ? (double)c->nnz / c->sM : 0.0));
+            break;
         case SDDMM_EXACT:
             if (c->dtype == SDDMM_BF16)
                 hipLaunchKernelGGL(k_exact<true>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
@@ -274,23 +376,23 @@ int enqueue_run(sddmm_ctx *c) {
         default: return fail(c, SDDMM_ERR_STATE, "no kernel for strategy %d", c->strategy);
     }
     HIP_TRY(c, hipGetLastError());
+    c->stats.kernels_launched = c->launches;
     return SDDMM_OK;
 }
 
 int do_plan(sddmm_ctx *c, int strategy) {
     int resolved = strategy;
     const bool csr_ok = c->have_rowptr;
-    if (strategy == SDDMM_AUTO) {
-        if (!csr_ok) resolved = SDDMM_FLAT;
-        else {
-            const double avg = c->sM ? (double)c->nnz / (double)c->sM : 0.0;
-            // whole-row waves pay off once a typical row fills a 64-entry chunk and
-            // no single row dominates the run time
-            const bool balanced = (double)c->pc.max_len <= 64.0 * std::max(avg, 1.0);
-            resolved = (avg >= 32.0 && balanced) ? SDDMM_ROW_WAVE : SDDMM_FLAT;
-        }
-    }
+    // without a row pointer (unsorted COO) only the flat kernels apply
+    if (strategy == SDDMM_AUTO && !csr_ok) resolved = SDDMM_FLAT;
     switch (resolved) {
+        case SDDMM_AUTO: {
+            c->ts = std::max(1, env_int("SDDMM_TS", 24));
+            c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+            int rc = classify_rows(c);
+            if (rc) return rc;
+            break;
+        }
         case SDDMM_FLAT:
         case SDDMM_EXACT: {
             int rc = ensure_rowidx(c);
@@ -298,9 +400,9 @@ int do_plan(sddmm_ctx *c, int strategy) {
             break;
         }
         case SDDMM_ROW_WAVE:
-            if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "ROW_WAVE needs row-sorted entries");
-            break;
         case SDDMM_SHORT_ROWS:
+            if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
+            break;
         case SDDMM_LDS_TILED:
         case SDDMM_MFMA_TILE:
             return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d is not available in this build", resolved);
@@ -317,6 +419,12 @@ void fill_model(sddmm_ctx *c) {
     s.strategy_used = c->strategy;
     s.nnz = c->nnz;
     s.rows_nonempty = (int64_t)c->pc.rows_nonempty;
+    if (c->strategy == SDDMM_AUTO) {
+        s.rows_short = (int64_t)c->pc.rows_short; s.rows_medium = (int64_t)c->pc.rows_medium;
+        s.rows_long = (int64_t)c->pc.rows_long;
+        s.nnz_short = (int64_t)c->pc.nnz_short; s.nnz_medium = (int64_t)c->pc.nnz_medium;
+        s.nnz_long = (int64_t)c->pc.nnz_long;
+    }
     const double e = (double)elem_size(c->dtype);
     s.flops = 2.0 * (double)c->nnz * (double)c->K;
     s.bytes_gathered = 4.0 * ((double)c->sM + 1.0) + 12.0 * (double)c->nnz +
@@ -596,7 +704,7 @@ int sddmm_run(sddmm_ctx *c) {
     float ms = 0.f;
     HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
     c->stats.run_ms = ms;
-    c->stats.kernels_launched = c->nnz ? 1 : 0;
+    c->stats.kernels_launched = c->launches;
     return SDDMM_OK;
 }
 

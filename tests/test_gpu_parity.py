@@ -19,7 +19,7 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 f32 = np.float32
 
-FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.EXACT]
+FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.EXACT]
 
 
 def _say(*a):
@@ -117,7 +117,7 @@ KS = [1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 31, 32, 33, 48, 64, 96, 100, 128, 160, 25
 def test_any_k(engine_factory, K):
     rng = np.random.default_rng(K)
     rowptr, col, val, A, B = _random_case(rng, 150, 130, K, 0.25)
-    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.EXACT):
+    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.AUTO, capi.EXACT):
         _say("K", K, capi.STRATEGY_NAMES[strategy])
         got, _ = run_csr(engine_factory, rowptr, col, val, A, B, 130, strategy)
         assert_parity(got, rowptr, col, val, A, B, exact=(strategy == capi.EXACT), what="K=%d" % K)
@@ -131,8 +131,10 @@ def test_strategies_agree_bitwise(engine_factory):
         a, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.FLAT)
         b, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.ROW_WAVE)
         c, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.AUTO)
+        d, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.SHORT_ROWS)
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
         np.testing.assert_array_equal(a.view(np.uint32), c.view(np.uint32))
+        np.testing.assert_array_equal(a.view(np.uint32), d.view(np.uint32))
 
 
 def test_edge_shapes(engine_factory):
@@ -213,9 +215,10 @@ def test_coo_sorted_and_unsorted(engine_factory):
     e = engine_factory()
     e.set_dense(A, B)
     e.set_coo(300, 200, rows[p], col[p], val[p])
-    with pytest.raises(capi.SddmmError) as ei:
-        e.plan(capi.ROW_WAVE)
-    assert ei.value.code == capi.ERR_UNSUPPORTED
+    for st in (capi.ROW_WAVE, capi.SHORT_ROWS):
+        with pytest.raises(capi.SddmmError) as ei:
+            e.plan(st)
+        assert ei.value.code == capi.ERR_UNSUPPORTED
     e.close()
 
 
@@ -290,8 +293,36 @@ def test_benchmark_shapes_scaled_down(engine_factory, name):
 @pytest.mark.parametrize("K", [32, 128])
 def test_bf16_inputs_gather_path(engine_factory, K):
     w = W.make("dense_tiles", "small", K=K)
-    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.EXACT):
+    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.AUTO, capi.EXACT):
         _say("bf16", K, capi.STRATEGY_NAMES[strategy])
         got, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A_bits, w.B_bits, w.N, strategy, capi.BF16)
         # products of bf16 values are exact in fp32, accumulation is fp32: the fp32 bar applies
         assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, rtol=1e-5, exact=(strategy == capi.EXACT), what="bf16")
+
+
+def test_auto_row_classes_and_segments(engine_factory):
+    """AUTO: rows below the short threshold go to the many-rows kernel, the rest to
+    wave-per-segment items; very long rows are cut into several segments."""
+    rng = np.random.default_rng(21)
+    M, N, K = 1000, 6000, 32
+    lens = rng.integers(0, 20, M)
+    lens[::50] = rng.integers(30, 300, len(lens[::50]))
+    lens[7] = 5000                                       # several segments
+    lens[500] = 0
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(N, l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.AUTO)
+    assert_parity(got, rowptr, col, val, A, B, what="auto classes")
+    assert st.strategy_used == capi.AUTO and st.kernels_launched == 1
+    ts, seg = 24, 2048
+    assert st.rows_short == np.count_nonzero((lens > 0) & (lens < ts))
+    assert st.nnz_short == lens[lens < ts].sum()
+    assert st.rows_long == np.count_nonzero(lens > seg) == 1
+    assert st.rows_medium == np.count_nonzero((lens >= ts) & (lens <= seg))
+    assert st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
+    assert st.rows_nonempty == np.count_nonzero(lens)
+    ref = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.FLAT)[0]
+    np.testing.assert_array_equal(got.view(np.uint32), ref.view(np.uint32))
