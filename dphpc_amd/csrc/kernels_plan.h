@@ -126,9 +126,12 @@ constexpr int SCAN_BLOCK = 256;
 constexpr int SCAN_ITEMS = 4;                       // rows per thread
 constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;  // rows per block
 
-__device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr, int64_t i, int M,
-                                                       int ts, int seg, unsigned int *len_out) {
-    if (i >= M) { *len_out = 0; return 0; }
+// strip_ntiles (may be null): rows of a strip that the dense-tile path owns count
+// as empty here
+__device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr,
+                                                       const unsigned int *__restrict__ strip_ntiles, int64_t i,
+                                                       int M, int ts, int seg, unsigned int *len_out) {
+    if (i >= M || (strip_ntiles && strip_ntiles[i >> 4] != 0)) { *len_out = 0; return 0; }
     const unsigned int len = (unsigned int)(rowptr[i + 1] - rowptr[i]);
     *len_out = len;
     return len >= (unsigned int)ts ? (len + seg - 1) / seg : 0u;
@@ -158,15 +161,16 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 }
 
 // pass 1: items per block of SCAN_TILE rows, plus the row statistics
-__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr, int M, int ts,
-                                                               int seg, unsigned int *__restrict__ block_sums,
+__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
+                                                               const unsigned int *__restrict__ strip_ntiles, int M,
+                                                               int ts, int seg, unsigned int *__restrict__ block_sums,
                                                                PlanCounters *pc) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int items = 0;
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        const unsigned int cnt = row_item_count(rowptr, base + q, M, ts, seg, &len);
+        const unsigned int cnt = row_item_count(rowptr, strip_ntiles, base + q, M, ts, seg, &len);
         items += cnt;
         if (len == 0) continue;
         if (cnt == 0) { ++r_short; n_short += len; }
@@ -188,9 +192,9 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__
     }
 }
 
-// pass 2: exclusive scan of the block sums in place (one workgroup), total -> pc->n_items
+// pass 2: exclusive scan of the block sums in place (one workgroup), total -> *total_out
 __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__restrict__ block_sums, int n,
-                                                                PlanCounters *pc) {
+                                                                unsigned long long *__restrict__ total_out) {
     unsigned int carry = 0;
     for (int base = 0; base < n; base += SCAN_BLOCK) {
         const int i = base + (int)threadIdx.x;
@@ -200,18 +204,20 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__
         if (i < n) block_sums[i] = carry + ex;
         carry += total;
     }
-    if (threadIdx.x == 0) pc->n_items = carry;
+    if (threadIdx.x == 0) *total_out = carry;
 }
 
 // pass 3: write the items
-__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr, int M, int ts,
-                                                               int seg, const unsigned int *__restrict__ block_offsets,
+__global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr,
+                                                               const unsigned int *__restrict__ strip_ntiles, int M,
+                                                               int ts, int seg,
+                                                               const unsigned int *__restrict__ block_offsets,
                                                                RowItem *__restrict__ items) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int cnt[SCAN_ITEMS], mine = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        cnt[q] = row_item_count(rowptr, base + q, M, ts, seg, &len);
+        cnt[q] = row_item_count(rowptr, strip_ntiles, base + q, M, ts, seg, &len);
         mine += cnt[q];
     }
     unsigned int total;

@@ -1,0 +1,258 @@
+// Dense-tile path: 16-row strips of S whose 16x16 tiles are well filled are
+// computed on the matrix cores, one MFMA accumulator per tile, instead of one
+// gathered B row per stored entry.
+//
+//   * a strip is rows [16*ti, 16*ti+16); a tile is the strip's entries whose
+//     column lies in [16*tj, 16*tj+16);
+//   * the classifier (k_tile_count / k_tile_fill, plan phase, device only) walks
+//     the sorted column lists of the 16 rows of a strip in step and emits one
+//     TileDesc per non-empty tile: for every row the CSR position of its first
+//     entry inside the tile and a 16-bit mask of the columns present;
+//   * a strip goes to this path as a whole (then every one of its entries is
+//     computed here, sparse tiles included) or not at all, so the gather kernels
+//     and this one never share a row;
+//   * k_tile computes the full 16x16 product A[strip rows] * B[tile cols]^T with
+//     fp32 accumulation (bf16: v_mfma_f32_16x16x32_bf16, fp32: v_mfma_f32_16x16x4_f32,
+//     both exact products of the stored inputs), multiplies by the S values and
+//     writes only the positions the masks name -- P keeps S's order.
+//
+// The B tile costs 16 rows per tile whatever its fill, a gathered entry costs one
+// row each: the tile path moves fewer bytes once a tile holds more than 16
+// entries, and far fewer at the 25-100 % fill it is used for.
+#pragma once
+#include "device_utils.h"
+#include "kernels_plan.h"
+
+namespace sddmm {
+
+struct alignas(16) TileDesc {
+    int32_t strip;      // 16-row strip index
+    int32_t tj;         // tile column: columns [16*tj, 16*tj+16)
+    int32_t pad[2];
+    int32_t off[16];    // per row: CSR position of the row's first entry in the tile
+    uint16_t mask[16];  // per row: bit c set <=> column 16*tj+c is stored
+};
+static_assert(sizeof(TileDesc) == 112, "TileDesc layout");
+
+// ---- 16-lane helpers (a strip is walked by 16 neighbouring lanes) -------------
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+}
+__device__ __forceinline__ int min16(int v) {
+    int o;
+    o = dpp_i32<DPP_QUAD_XOR1>(v); v = o < v ? o : v;
+    o = dpp_i32<DPP_QUAD_XOR2>(v); v = o < v ? o : v;
+    o = dpp_i32<DPP_ROW_HALF_MIRROR>(v); v = o < v ? o : v;
+    o = dpp_i32<DPP_ROW_MIRROR>(v); v = o < v ? o : v;
+    return v;
+}
+__device__ __forceinline__ int sum16(int v) {
+    v += dpp_i32<DPP_QUAD_XOR1>(v);
+    v += dpp_i32<DPP_QUAD_XOR2>(v);
+    v += dpp_i32<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_i32<DPP_ROW_MIRROR>(v);
+    return v;
+}
+
+// Walks the tiles of one strip in increasing tile column.  All 16 lanes of the
+// strip call on_tile(tj, first, mask) together; `first` / `mask` are this lane's
+// row's first position and column mask in the tile (mask 0: row absent).
+// Returns false in a lane whose row is not strictly increasing in column.
+template <class F>
+__device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M,
+                                           int64_t strip, int sub, F &&on_tile) {
+    const int64_t row = strip * 16 + sub;
+    int p = 0, end = 0;
+    if (row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
+    bool sorted = true;
+    int prev = -1;
+    int c = p < end ? col[p] : -1;
+    while (true) {
+        const int mine = p < end ? (c >> 4) : INT32_MAX;
+        const int t = min16(mine);
+        if (t == INT32_MAX) break;
+        const int first = p;
+        unsigned int mask = 0;
+        while (p < end && (c >> 4) == t) {
+            if (c <= prev) sorted = false;
+            prev = c;
+            mask |= 1u << (c & 15);
+            ++p;
+            c = p < end ? col[p] : -1;
+        }
+        on_tile(t, first, mask);
+    }
+    return sorted;
+}
+
+// pass 1: tiles and entries per strip; a strip qualifies when all its rows are
+// sorted and it holds at least min_fill entries per tile on average.
+// strip_ntiles[s] = number of tiles (0: strip stays on the gather kernels).
+__global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ rowptr,
+                                                    const int32_t *__restrict__ col, int M, int64_t n_strips,
+                                                    int min_fill, unsigned int *__restrict__ strip_ntiles,
+                                                    PlanCounters *pc) {
+    const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    if (strip >= n_strips) return;   // whole 16-lane rows leave together
+    int tiles = 0, entries = 0;
+    const bool sorted = walk_strip(rowptr, col, M, strip, sub, [&](int, int, unsigned int mask) {
+        ++tiles;
+        entries += __builtin_popcount(mask);
+    });
+    const int all_entries = sum16(entries);
+    const int unsorted = sum16(sorted ? 0 : 1);
+    const bool take = unsorted == 0 && tiles > 0 && (int64_t)all_entries >= (int64_t)min_fill * tiles;
+    if (sub == 0) {
+        strip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
+        if (take) {
+            atomicAdd(&pc->spare[0], (unsigned long long)tiles);        // tiles on the MFMA path
+            atomicAdd(&pc->spare[1], (unsigned long long)all_entries);  // entries they cover
+        }
+    }
+}
+
+// pass 2 (after the exclusive scan of strip_ntiles into strip_off): descriptors
+__global__ __launch_bounds__(256) void k_tile_fill(const int32_t *__restrict__ rowptr,
+                                                   const int32_t *__restrict__ col, int M, int64_t n_strips,
+                                                   const unsigned int *__restrict__ strip_ntiles,
+                                                   const unsigned int *__restrict__ strip_off,
+                                                   TileDesc *__restrict__ tiles) {
+    const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    if (strip >= n_strips) return;
+    if (strip_ntiles[strip] == 0) return;
+    int64_t at = strip_off[strip];
+    (void)walk_strip(rowptr, col, M, strip, sub, [&](int tj, int first, unsigned int mask) {
+        TileDesc *d = tiles + at;
+        d->off[sub] = first;
+        d->mask[sub] = (uint16_t)mask;
+        if (sub == 0) { d->strip = (int32_t)strip; d->tj = tj; d->pad[0] = 0; d->pad[1] = 0; }
+        ++at;
+    });
+}
+
+// generic exclusive scan of n unsigned ints: block sums, then apply
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_sums(const unsigned int *__restrict__ in, int64_t n,
+                                                          unsigned int *__restrict__ block_sums) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    unsigned int mine = 0;
+    for (int q = 0; q < SCAN_ITEMS; ++q) mine += base + q < n ? in[base + q] : 0u;
+    unsigned int total;
+    (void)block_exclusive_scan(mine, &total);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_apply(const unsigned int *__restrict__ in, int64_t n,
+                                                           const unsigned int *__restrict__ block_offsets,
+                                                           unsigned int *__restrict__ out) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    unsigned int v[SCAN_ITEMS], mine = 0;
+    for (int q = 0; q < SCAN_ITEMS; ++q) { v[q] = base + q < n ? in[base + q] : 0u; mine += v[q]; }
+    unsigned int total;
+    unsigned int at = block_offsets[blockIdx.x] + block_exclusive_scan(mine, &total);
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        if (base + q < n) out[base + q] = at;
+        at += v[q];
+    }
+}
+
+// ---- the MFMA kernel ------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+// One wavefront computes `tiles_per_wave` consecutive tiles.  Operand layout of
+// both MFMA shapes used: lane l supplies row (l & 15) of its operand and the k
+// positions selected by (l >> 4); the result register i of lane l is row
+// 4*(l >> 4) + i, column (l & 15).  A and B are read in 16-byte units: in load
+// step s lane l reads unit 4*s + (l >> 4) of its row, so the four lane groups
+// cover 64 contiguous bytes of each of 16 rows per instruction; which k positions
+// end up in which MFMA does not matter as long as A and B agree.
+// STEPS = row bytes / 64.  The A panel of the current strip stays in registers;
+// the next tile's descriptor and B units are requested before the current tile's
+// MFMAs are issued.
+template <bool BF16, int STEPS>
+__global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                                const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                int tiles_per_wave, const float *__restrict__ sval,
+                                                float *__restrict__ P, int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
+    int64_t t = w * tiles_per_wave;
+    if (t >= n_tiles) return;
+    int64_t t_end = t + tiles_per_wave;
+    t_end = t_end < n_tiles ? t_end : n_tiles;
+    const int lane = lane_id();
+    const int r16 = lane & 15, q = lane >> 4;
+    constexpr uint32_t ROW_BYTES = STEPS * 64;
+    const uint4 *__restrict__ Au = (const uint4 *)A;
+    const uint4 *__restrict__ Bu = (const uint4 *)B;
+
+    struct Pending {
+        int strip, tj;
+        int4 off;
+        uint2 mask;
+        uint4 b[STEPS];
+    };
+    auto fetch = [&](int64_t ti, Pending &pd) {
+        const TileDesc *d = tiles + ti;
+        pd.strip = __builtin_amdgcn_readfirstlane(d->strip);
+        pd.tj = __builtin_amdgcn_readfirstlane(d->tj);
+        pd.off = *(const int4 *)&d->off[q * 4];
+        pd.mask = *(const uint2 *)&d->mask[q * 4];
+        int64_t brow = (int64_t)pd.tj * 16 + r16;
+        brow = brow < N ? brow : N - 1;   // columns past N are never in a mask
+        const uint4 *src = Bu + brow * (ROW_BYTES / 16) + q;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) pd.b[s] = src[s * 4];
+    };
+
+    Pending cur, nxt;
+    fetch(t, cur);
+    int cur_strip = -1;
+    uint4 a[STEPS];
+    for (; t < t_end; ++t) {
+        if (cur.strip != cur_strip) {
+            cur_strip = cur.strip;
+            int64_t arow = (int64_t)cur_strip * 16 + r16;
+            arow = arow < M ? arow : M - 1;   // rows past M are never in a mask
+            const uint4 *src = Au + arow * (ROW_BYTES / 16) + q;
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
+        }
+        const int64_t tn = t + 1 < t_end ? t + 1 : t;
+        fetch(tn, nxt);
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            if constexpr (BF16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
+                                                              __builtin_bit_cast(bf16x8_t, cur.b[s]), acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
+                                                           __builtin_bit_cast(float, cur.b[s].x), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].y),
+                                                           __builtin_bit_cast(float, cur.b[s].y), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].z),
+                                                           __builtin_bit_cast(float, cur.b[s].z), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].w),
+                                                           __builtin_bit_cast(float, cur.b[s].w), acc, 0, 0, 0);
+            }
+        }
+        // scale by S and scatter: row 4*q+i, column r16
+        const int offs[4] = {cur.off.x, cur.off.y, cur.off.z, cur.off.w};
+        const unsigned int masks[4] = {cur.mask.x & 0xFFFFu, cur.mask.x >> 16, cur.mask.y & 0xFFFFu, cur.mask.y >> 16};
+        const unsigned int below = (1u << r16) - 1u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if ((masks[i] >> r16) & 1u) {
+                const int pos = offs[i] + __builtin_popcount(masks[i] & below);
+                P[pos] = acc[i] * sval[pos];
+            }
+        }
+        cur = nxt;
+    }
+}
+
+}  // namespace sddmm

@@ -15,6 +15,7 @@
 
 #include "kernels_gather.h"
 #include "kernels_plan.h"
+#include "kernels_tile.h"
 
 using namespace sddmm;
 
@@ -55,6 +56,13 @@ struct sddmm_ctx {
     int64_t block_sums_cap = 0;
     int64_t rows_short = 0;
     int launches = 0;
+    // dense-tile (MFMA) path
+    unsigned int *d_strip_ntiles = nullptr, *d_strip_off = nullptr;
+    int64_t strips_cap = 0;
+    TileDesc *d_tiles = nullptr;
+    int64_t n_tiles = 0, tiles_cap = 0, nnz_tiles = 0;
+    int tile_steps = 0, tiles_per_wave = 8;
+    bool tiles_active = false;       // d_strip_ntiles describes the current pattern
 };
 
 namespace {
@@ -108,7 +116,12 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->dP);
     dfree(c->d_items);
     dfree(c->d_block_sums);
+    dfree(c->d_strip_ntiles);
+    dfree(c->d_strip_off);
+    dfree(c->d_tiles);
     c->items_cap = c->block_sums_cap = c->n_items = 0;
+    c->strips_cap = c->tiles_cap = c->n_tiles = c->nnz_tiles = 0;
+    c->tiles_active = false;
     c->d_col = nullptr; c->d_sval = nullptr; c->d_rowptr = nullptr; c->d_rowidx = nullptr;
     c->own_sparse = c->own_rowptr = c->own_rowidx = false;
     c->have_sparse = c->have_rowptr = false;
@@ -260,8 +273,9 @@ void launch_auto(sddmm_ctx *c) {
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
         hipLaunchKernelGGL((k_auto<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
-                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
-                           c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
+                           (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
+                           (const unsigned int *)(c->tiles_active ? c->d_strip_ntiles : nullptr), c->d_col, c->d_sval,
+                           c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
     });
 }
 
@@ -286,10 +300,11 @@ int classify_rows(sddmm_ctx *c) {
     c->pc = fresh;
     HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
     if (nb > 0) {
-        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, c->sM,
-                           c->ts, c->seg, c->d_block_sums, c->d_pc);
+        const unsigned int *strips = c->tiles_active ? c->d_strip_ntiles : nullptr;
+        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, strips,
+                           c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc);
         hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
-                           c->d_pc);
+                           &c->d_pc->n_items);
         HIP_TRY(c, hipGetLastError());
     }
     int rc = fetch_counters(c);
@@ -304,11 +319,92 @@ int classify_rows(sddmm_ctx *c) {
         c->items_cap = c->n_items;
     }
     if (c->n_items > 0) {
-        hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, c->sM,
-                           c->ts, c->seg, c->d_block_sums, c->d_items);
+        hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+                           c->tiles_active ? c->d_strip_ntiles : nullptr, c->sM, c->ts, c->seg, c->d_block_sums,
+                           c->d_items);
         HIP_TRY(c, hipGetLastError());
     }
     return SDDMM_OK;
+}
+
+// Dense-tile classifier.  min_fill = average stored entries per 16x16 tile a strip
+// needs to be taken.  Leaves tiles_active false when the path does not apply
+// (no row pointer, row size not a multiple of 64 bytes, nothing qualifies).
+int plan_tiles(sddmm_ctx *c, int min_fill) {
+    c->tiles_active = false;
+    c->n_tiles = c->nnz_tiles = 0;
+    if (!c->have_rowptr || c->nnz == 0) return SDDMM_OK;
+    const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
+    if (row_bytes % 64) return SDDMM_OK;
+    const int steps = (int)(row_bytes / 64);
+    if (steps != 1 && steps != 2 && steps != 4 && steps != 8 && steps != 16) return SDDMM_OK;
+    c->tile_steps = steps;
+    const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
+    if (n_strips > c->strips_cap) {
+        dfree(c->d_strip_ntiles);
+        dfree(c->d_strip_off);
+        ALLOC_TRY(c, c->d_strip_ntiles, (size_t)n_strips * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_strip_off, (size_t)n_strips * sizeof(unsigned int));
+        c->strips_cap = n_strips;
+    }
+    const int64_t nb = (n_strips + SCAN_TILE - 1) / SCAN_TILE;
+    if (nb > c->block_sums_cap) {
+        dfree(c->d_block_sums);
+        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
+        c->block_sums_cap = nb;
+    }
+    c->pc.spare[0] = c->pc.spare[1] = c->pc.spare[2] = 0;
+    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
+    const unsigned walk_grid = (unsigned)((n_strips * 16 + 255) / 256);
+    hipLaunchKernelGGL(k_tile_count, dim3(walk_grid), dim3(256), 0, c->stream, c->d_rowptr, c->d_col, c->sM, n_strips,
+                       min_fill, c->d_strip_ntiles, c->d_pc);
+    hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_strip_ntiles, n_strips,
+                       c->d_block_sums);
+    hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
+                       &c->d_pc->spare[2]);
+    hipLaunchKernelGGL(k_scan_apply, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_strip_ntiles, n_strips,
+                       c->d_block_sums, c->d_strip_off);
+    HIP_TRY(c, hipGetLastError());
+    int rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_tiles = (int64_t)c->pc.spare[0];
+    c->nnz_tiles = (int64_t)c->pc.spare[1];
+    if ((int64_t)c->pc.spare[2] != c->n_tiles) return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
+    if (c->n_tiles == 0) return SDDMM_OK;
+    if (c->n_tiles > c->tiles_cap) {
+        dfree(c->d_tiles);
+        ALLOC_TRY(c, c->d_tiles, (size_t)c->n_tiles * sizeof(TileDesc));
+        c->tiles_cap = c->n_tiles;
+    }
+    hipLaunchKernelGGL(k_tile_fill, dim3(walk_grid), dim3(256), 0, c->stream, c->d_rowptr, c->d_col, c->sM, n_strips,
+                       c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
+    HIP_TRY(c, hipGetLastError());
+    c->tiles_active = true;
+    c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 8));
+    return SDDMM_OK;
+}
+
+template <bool BF16, int STEPS>
+void launch_tile_t(sddmm_ctx *c) {
+    const int64_t waves = (c->n_tiles + c->tiles_per_wave - 1) / c->tiles_per_wave;
+    const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    hipLaunchKernelGGL((k_tile<BF16, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                       (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const TileDesc *)c->d_tiles, c->n_tiles,
+                       c->tiles_per_wave, (const float *)c->d_sval, c->dP, nblocks);
+}
+template <bool BF16>
+void launch_tile_steps(sddmm_ctx *c) {
+    switch (c->tile_steps) {
+        case 1: launch_tile_t<BF16, 1>(c); break;
+        case 2: launch_tile_t<BF16, 2>(c); break;
+        case 4: launch_tile_t<BF16, 4>(c); break;
+        case 8: launch_tile_t<BF16, 8>(c); break;
+        default: launch_tile_t<BF16, 16>(c); break;
+    }
+}
+void launch_tiles(sddmm_ctx *c) {
+    if (c->dtype == SDDMM_BF16) launch_tile_steps<true>(c);
+    else launch_tile_steps<false>(c);
 }
 
 int ensure_rowidx(sddmm_ctx *c) {
@@ -357,8 +453,10 @@ int enqueue_run(sddmm_ctx *c) {
     c->launches = 1;
     switch (c->strategy) {
         case SDDMM_AUTO:
-            if (c->rows_short == 0 && c->n_items == 0) { c->launches = 0; break; }
-            launch_auto(c);
+        case SDDMM_MFMA_TILE:
+            c->launches = 0;
+            if (c->tiles_active && c->n_tiles > 0) { launch_tiles(c); ++c->launches; }
+            if (c->rows_short > 0 || c->n_items > 0) { launch_auto(c); ++c->launches; }
             break;
         case SDDMM_FLAT: launch_flat(c); break;
         case SDDMM_ROW_WAVE: launch_row_wave(c, nullptr, c->sM); break;
@@ -386,10 +484,16 @@ int do_plan(sddmm_ctx *c, int strategy) {
     // without a row pointer (unsorted COO) only the flat kernels apply
     if (strategy == SDDMM_AUTO && !csr_ok) resolved = SDDMM_FLAT;
     switch (resolved) {
-        case SDDMM_AUTO: {
+        case SDDMM_AUTO:
+        case SDDMM_MFMA_TILE: {
+            // strips first (they take whole rows away from the row classes), then rows;
+            // MFMA_TILE takes every sorted strip, AUTO only the well-filled ones
+            if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
+            int rc = plan_tiles(c, resolved == SDDMM_MFMA_TILE ? 1 : std::max(1, env_int("SDDMM_TILE_FILL", 32)));
+            if (rc) return rc;
             c->ts = std::max(1, env_int("SDDMM_TS", 24));
             c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
-            int rc = classify_rows(c);
+            rc = classify_rows(c);
             if (rc) return rc;
             break;
         }
@@ -404,7 +508,6 @@ int do_plan(sddmm_ctx *c, int strategy) {
             if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
             break;
         case SDDMM_LDS_TILED:
-        case SDDMM_MFMA_TILE:
             return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d is not available in this build", resolved);
         default: return fail(c, SDDMM_ERR_INVALID, "unknown strategy %d", strategy);
     }
@@ -419,7 +522,9 @@ void fill_model(sddmm_ctx *c) {
     s.strategy_used = c->strategy;
     s.nnz = c->nnz;
     s.rows_nonempty = (int64_t)c->pc.rows_nonempty;
-    if (c->strategy == SDDMM_AUTO) {
+    if (c->strategy == SDDMM_AUTO || c->strategy == SDDMM_MFMA_TILE) {
+        s.mfma_tiles = c->tiles_active ? c->n_tiles : 0;
+        s.nnz_mfma = c->tiles_active ? c->nnz_tiles : 0;
         s.rows_short = (int64_t)c->pc.rows_short; s.rows_medium = (int64_t)c->pc.rows_medium;
         s.rows_long = (int64_t)c->pc.rows_long;
         s.nnz_short = (int64_t)c->pc.nnz_short; s.nnz_medium = (int64_t)c->pc.nnz_medium;

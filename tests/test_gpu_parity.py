@@ -19,7 +19,7 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 f32 = np.float32
 
-FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.EXACT]
+FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.MFMA_TILE, capi.EXACT]
 
 
 def _say(*a):
@@ -124,13 +124,15 @@ def test_any_k(engine_factory, K):
 
 
 def test_strategies_agree_bitwise(engine_factory):
-    # same per-entry arithmetic in every gather kernel
+    # same per-entry arithmetic in every gather kernel (density below the tile
+    # path's threshold, so that AUTO is made of gather kernels only)
     rng = np.random.default_rng(77)
     for K in (32, 64, 20, 7, 128):
-        rowptr, col, val, A, B = _random_case(rng, 400, 300, K, 0.2)
+        rowptr, col, val, A, B = _random_case(rng, 400, 300, K, 0.08)
         a, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.FLAT)
         b, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.ROW_WAVE)
-        c, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.AUTO)
+        c, st = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.AUTO)
+        assert st.mfma_tiles == 0
         d, _ = run_csr(engine_factory, rowptr, col, val, A, B, 300, capi.SHORT_ROWS)
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
         np.testing.assert_array_equal(a.view(np.uint32), c.view(np.uint32))
@@ -288,6 +290,8 @@ def test_benchmark_shapes_scaled_down(engine_factory, name):
         assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, exact=(strategy == capi.EXACT), what=name)
         assert st.flops == 2.0 * w.nnz * w.K
         assert st.bytes_gathered == w.bytes_gathered()
+        if strategy == capi.AUTO and name in ("power_law", "mixed_density", "small_uniform"):
+            assert st.mfma_tiles == 0          # nothing there is dense enough for the tile path
 
 
 @pytest.mark.parametrize("K", [32, 128])
@@ -324,5 +328,89 @@ def test_auto_row_classes_and_segments(engine_factory):
     assert st.rows_medium == np.count_nonzero((lens >= ts) & (lens <= seg))
     assert st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
     assert st.rows_nonempty == np.count_nonzero(lens)
+    assert st.mfma_tiles == 0
     ref = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.FLAT)[0]
     np.testing.assert_array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+# ---- dense-tile (MFMA) path ------------------------------------------------------
+def _tile_count(rowptr, col, M):
+    rows = np.repeat(np.arange(M), np.diff(rowptr))
+    return len(np.unique((rows // 16).astype(np.int64) * (1 << 32) + (col // 16)))
+
+
+@pytest.mark.parametrize("K", [32, 128, 512])
+def test_mfma_tiles_bf16(engine_factory, K):
+    """bf16 inputs, fully dense 16x16 tiles.  Products of bf16 values are exact in
+    fp32 and the accumulator is fp32, so the result is held to the fp32 bar
+    (1e-5 with the magnitude floor), well inside the 1e-2 allowed for this path."""
+    w = W.make("dense_tiles", "small", K=K)
+    for strategy in (capi.AUTO, capi.MFMA_TILE):
+        _say("mfma bf16", K, capi.STRATEGY_NAMES[strategy])
+        got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A_bits, w.B_bits, w.N, strategy, capi.BF16)
+        assert st.mfma_tiles == w.meta["tiles"] and st.nnz_mfma == w.nnz
+        assert st.kernels_launched == 1
+        assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, rtol=1e-5, what="mfma bf16 K=%d" % K)
+
+
+@pytest.mark.parametrize("K", [16, 32, 64, 128, 256])
+def test_mfma_tiles_fp32(engine_factory, K):
+    w = W.make("dense_tiles", "small", K=K, bf16=False)
+    for strategy in (capi.AUTO, capi.MFMA_TILE):
+        _say("mfma f32", K, capi.STRATEGY_NAMES[strategy])
+        got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, strategy)
+        assert st.mfma_tiles == w.meta["tiles"] and st.nnz_mfma == w.nnz
+        assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="mfma f32 K=%d" % K)
+
+
+def test_tiles_partial_fill_ragged_edges_and_mixed_strips(engine_factory):
+    """Strips of every kind in one matrix: full tiles, partly filled tiles, 8x8
+    blocks, strips too sparse for the tile path, an unsorted row (its strip must
+    stay on the gather kernels), M and N not multiples of 16."""
+    rng = np.random.default_rng(33)
+    M, N, K = 16 * 9 + 5, 16 * 13 + 7, 32
+    dense = np.zeros((M, N), bool)
+    dense[0:16, 32:64] = True                                  # strip 0: two full tiles
+    dense[16:32, :] = rng.random((16, N)) < 0.5                # strip 1: half filled everywhere
+    for b in range(4):                                         # strip 2: 8x8 blocks
+        dense[32 + 8 * (b % 2):40 + 8 * (b % 2), 16 * b + 8 * (b % 2):16 * b + 8 * (b % 2) + 8] = True
+    dense[48:64, :] = rng.random((16, N)) < 0.02               # strip 3: sparse -> gather
+    dense[64:80, 100:180] = rng.random((16, 80)) < 0.7         # strip 4: unsorted row below
+    dense[80:96, N - 7:] = True                                # strip 5: last, partial tile column
+    dense[128:, 0:40] = rng.random((M - 128, 40)) < 0.6        # last strip has only 5+16 rows
+    r, c = np.nonzero(dense)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    s, e = rowptr[70], rowptr[71]
+    assert e - s >= 2
+    col[s], col[s + 1] = col[s + 1], col[s]                    # row 70 no longer sorted
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    for strategy in (capi.AUTO, capi.MFMA_TILE):
+        got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, strategy)
+        assert_parity(got, rowptr, col, val, A, B, what="mixed strips")
+        assert st.mfma_tiles > 0 and 0 < st.nnz_mfma < len(col)
+        assert st.kernels_launched == 2
+    rows = np.repeat(np.arange(M), np.diff(rowptr))
+    forced = rows // 16 != 4                                   # MFMA_TILE: every strip but the unsorted one
+    assert st.nnz_mfma == np.count_nonzero(forced)
+    assert st.mfma_tiles == _tile_count(rowptr, col, M) - len(np.unique(col[rows // 16 == 4] // 16))
+    # AUTO leaves the sparse strip to the gather kernels as well
+    _, st_auto = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.AUTO)
+    assert st_auto.nnz_mfma == np.count_nonzero(forced & (rows // 16 != 3))
+
+
+def test_tile_path_not_applicable_falls_back_to_gather(engine_factory):
+    # K*4 not a multiple of 64 bytes, and bf16 with K=8: everything on the gather kernels
+    rng = np.random.default_rng(34)
+    w = W.make("dense_tiles", "small", K=24, bf16=False)
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.MFMA_TILE)
+    assert st.mfma_tiles == 0 and st.nnz_mfma == 0
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B)
+
+
+def test_fem_blocks_take_the_tile_path(engine_factory):
+    w = W.make("fem_banded", "small")
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
+    assert st.nnz_mfma == w.nnz and st.mfma_tiles == _tile_count(w.rowptr, w.col, w.M)
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem tiles")
