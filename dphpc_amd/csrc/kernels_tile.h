@@ -168,9 +168,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // step s lane l reads unit 4*s + (l >> 4) of its row, so the four lane groups
 // cover 64 contiguous bytes of each of 16 rows per instruction; which k positions
 // end up in which MFMA does not matter as long as A and B agree.
-// STEPS = row bytes / 64.  The A panel of the current strip stays in registers;
-// the next tile's descriptor and B units are requested before the current tile's
-// MFMAs are issued.
+// STEPS = row bytes / 64.
+//
+// Software pipeline, three tiles deep, every load unconditional so that the wait
+// counts stay exact (loads return in issue order):
+//   iteration t issues   B rows + S values of tile t+1   (needs descriptor t+1)
+//                        descriptor of tile t+2
+//   and then computes    MFMAs of tile t, scale, scatter (operands landed during t-1)
+// The A panel of the current strip stays in registers and is reloaded only when
+// the strip changes (a wave-uniform branch placed before the iteration's loads).
 template <bool BF16, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
@@ -183,75 +189,97 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
     if (t >= n_tiles) return;
     int64_t t_end = t + tiles_per_wave;
     t_end = t_end < n_tiles ? t_end : n_tiles;
+    const int64_t t_last = t_end - 1;
     const int lane = lane_id();
     const int r16 = lane & 15, q = lane >> 4;
-    constexpr uint32_t ROW_BYTES = STEPS * 64;
+    constexpr uint32_t ROW_UNITS = STEPS * 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
+    const unsigned int below = (1u << r16) - 1u;
 
-    struct Pending {
+    struct Desc {
         int strip, tj;
         int4 off;
         uint2 mask;
-        uint4 b[STEPS];
     };
-    auto fetch = [&](int64_t ti, Pending &pd) {
+    struct Oper {
+        uint4 b[STEPS];
+        float s[4];
+        int pos[4];
+        unsigned int act;   // bit i: result register i is a stored entry
+    };
+    auto load_desc = [&](int64_t ti) {
+        ti = ti < t_last ? ti : t_last;
         const TileDesc *d = tiles + ti;
-        pd.strip = __builtin_amdgcn_readfirstlane(d->strip);
-        pd.tj = __builtin_amdgcn_readfirstlane(d->tj);
-        pd.off = *(const int4 *)&d->off[q * 4];
-        pd.mask = *(const uint2 *)&d->mask[q * 4];
-        int64_t brow = (int64_t)pd.tj * 16 + r16;
+        Desc r;
+        r.strip = d->strip;
+        r.tj = d->tj;
+        r.off = *(const int4 *)&d->off[q * 4];
+        r.mask = *(const uint2 *)&d->mask[q * 4];
+        return r;
+    };
+    auto load_oper = [&](const Desc &d) {
+        Oper o;
+        int64_t brow = (int64_t)d.tj * 16 + r16;
         brow = brow < N ? brow : N - 1;   // columns past N are never in a mask
-        const uint4 *src = Bu + brow * (ROW_BYTES / 16) + q;
+        const uint4 *src = Bu + brow * ROW_UNITS + q;
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) pd.b[s] = src[s * 4];
+        for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
+        const int offs[4] = {d.off.x, d.off.y, d.off.z, d.off.w};
+        const unsigned int masks[4] = {d.mask.x & 0xFFFFu, d.mask.x >> 16, d.mask.y & 0xFFFFu, d.mask.y >> 16};
+        o.act = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool on = (masks[i] >> r16) & 1u;
+            o.act |= on ? (1u << i) : 0u;
+            // position of (row 4q+i, column r16) in the CSR arrays; entry 0 when absent
+            o.pos[i] = on ? offs[i] + __builtin_popcount(masks[i] & below) : 0;
+            o.s[i] = sval[o.pos[i]];
+        }
+        return o;
     };
 
-    Pending cur, nxt;
-    fetch(t, cur);
+    Desc d_cur = load_desc(t);
+    Oper o_cur = load_oper(d_cur);
+    Desc d_nxt = load_desc(t + 1);
     int cur_strip = -1;
     uint4 a[STEPS];
     for (; t < t_end; ++t) {
-        if (cur.strip != cur_strip) {
-            cur_strip = cur.strip;
-            int64_t arow = (int64_t)cur_strip * 16 + r16;
+        const int strip = __builtin_amdgcn_readfirstlane(d_cur.strip);
+        if (strip != cur_strip) {
+            cur_strip = strip;
+            int64_t arow = (int64_t)strip * 16 + r16;
             arow = arow < M ? arow : M - 1;   // rows past M are never in a mask
-            const uint4 *src = Au + arow * (ROW_BYTES / 16) + q;
+            const uint4 *src = Au + arow * ROW_UNITS + q;
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
         }
-        const int64_t tn = t + 1 < t_end ? t + 1 : t;
-        fetch(tn, nxt);
+        const Oper o_nxt = load_oper(d_nxt);
+        const Desc d_nn = load_desc(t + 2);
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             if constexpr (BF16) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
-                                                              __builtin_bit_cast(bf16x8_t, cur.b[s]), acc, 0, 0, 0);
+                                                              __builtin_bit_cast(bf16x8_t, o_cur.b[s]), acc, 0, 0, 0);
             } else {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
-                                                           __builtin_bit_cast(float, cur.b[s].x), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, o_cur.b[s].x), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].y),
-                                                           __builtin_bit_cast(float, cur.b[s].y), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, o_cur.b[s].y), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].z),
-                                                           __builtin_bit_cast(float, cur.b[s].z), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, o_cur.b[s].z), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].w),
-                                                           __builtin_bit_cast(float, cur.b[s].w), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, o_cur.b[s].w), acc, 0, 0, 0);
             }
         }
-        // scale by S and scatter: row 4*q+i, column r16
-        const int offs[4] = {cur.off.x, cur.off.y, cur.off.z, cur.off.w};
-        const unsigned int masks[4] = {cur.mask.x & 0xFFFFu, cur.mask.x >> 16, cur.mask.y & 0xFFFFu, cur.mask.y >> 16};
-        const unsigned int below = (1u << r16) - 1u;
+        // scale by S and scatter: result register i is row 4*q+i, column r16
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if ((masks[i] >> r16) & 1u) {
-                const int pos = offs[i] + __builtin_popcount(masks[i] & below);
-                P[pos] = acc[i] * sval[pos];
-            }
-        }
-        cur = nxt;
+        for (int i = 0; i < 4; ++i)
+            if ((o_cur.act >> i) & 1u) P[o_cur.pos[i]] = acc[i] * o_cur.s[i];
+        o_cur = o_nxt;
+        d_cur = d_nxt;
+        d_nxt = d_nn;
     }
 }
 
