@@ -38,6 +38,7 @@ class Stats(C.Structure):
         ("nnz_short", C.c_int64), ("nnz_medium", C.c_int64), ("nnz_long", C.c_int64),
         ("mfma_tiles", C.c_int64), ("nnz_mfma", C.c_int64), ("cols_touched", C.c_int64),
         ("flops", C.c_double), ("bytes_gathered", C.c_double),
+        ("panels", C.c_int64), ("nnz_panel", C.c_int64),
     ]
 
     def as_dict(self):

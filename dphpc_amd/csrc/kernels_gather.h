@@ -282,7 +282,7 @@ __device__ __forceinline__ void row_segment_body(const void *__restrict__ A, con
 template <class L>
 __device__ __forceinline__ void short_rows_body(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                 const int32_t *__restrict__ rowptr,
-                                                const unsigned int *__restrict__ strip_ntiles,
+                                                const unsigned char *__restrict__ owner8,
                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
                                                 float *__restrict__ P, int M, int ts, int64_t r0, int rpw, int lane) {
     using U = typename L::U;
@@ -292,8 +292,8 @@ __device__ __forceinline__ void short_rows_body(const void *__restrict__ A, cons
         rs = rowptr[r0 + lane];
         len = rowptr[r0 + lane + 1] - rs;
         if (len >= ts) len = 0;
-        // rows of a strip owned by the dense-tile path
-        if (strip_ntiles && strip_ntiles[(r0 + lane) >> 4] != 0) len = 0;
+        // rows computed by the dense-tile or the row-panel path
+        if (owner8 && owner8[(r0 + lane) >> 3] != 0) len = 0;
     }
     int incl = len;
     for (int o = 1; o < WAVE; o <<= 1) {
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(BLOCK) void k_short_rows(const void *__restrict__ A
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                 const int32_t *__restrict__ rowptr,
-                                                const unsigned int *__restrict__ strip_ntiles,
+                                                const unsigned char *__restrict__ owner8,
                                                 const int32_t *__restrict__ col,
                                                 const float *__restrict__ sval, float *__restrict__ P, int M,
                                                 int ts, int rpw, int64_t short_blocks,
@@ -423,7 +423,147 @@ __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, cons
         const int64_t sb = blk - items_before;
         const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
         if (r0 >= M) return;
-        short_rows_body<L>(A, B, KU, rowptr, strip_ntiles, col, sval, P, M, ts, r0, rpw, lane_id());
+        short_rows_body<L>(A, B, KU, rowptr, owner8, col, sval, P, M, ts, r0, rpw, lane_id());
+    }
+}
+
+// ---------------------------------------------------------------------------
+// ROW PANEL: 8 consecutive rows with the same column list (the 8 rows of a dense
+// 8x8-block row of a finite-element matrix, the halves of a 16-row dense tile
+// strip).  One wavefront per work item = entries [start,end) of the shared list.
+// The column indices are read once for the 8 rows and every gathered B unit is
+// multiplied with the units of all 8 A rows, which stay in registers: one eighth
+// of the gather traffic of the per-row kernels.  Lane (g, j) computes, in step t,
+// column t*8+g of the chunk for all 8 rows and keeps row j's total, so S values
+// and P are accessed as 8 runs of 8 consecutive floats per instruction.
+// Needs the 8-lanes-per-entry layout with no masked unit (K*elem a multiple of 128).
+constexpr int PANEL_ROWS = 8;
+// Register budget: forcing more than 2 workgroups per CU makes the compiler spill
+// the A rows (measured 3x slower on MI355X), so the kernel runs at 2 waves per
+// SIMD and hides latency with its own software pipeline instead.
+#ifndef SDDMM_PANEL_OCC
+#define SDDMM_PANEL_OCC 2
+#endif
+
+template <class L>
+__global__ __launch_bounds__(BLOCK, SDDMM_PANEL_OCC) void k_panel(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                 const int32_t *__restrict__ rowptr,
+                                                 const int32_t *__restrict__ col,
+                                                 const float *__restrict__ sval, float *__restrict__ P,
+                                                 const RowItem *__restrict__ items, int64_t n_items,
+                                                 int64_t nblocks) {
+    using U = typename L::U;
+    using T = typename U::T;
+    static_assert(L::LPN == 8 && L::FULLK && !L::LONG, "row panels use the 8-lane full-K layout");
+    constexpr int UPL = L::UPL;
+    using O = typename Off<L::WIDE>::T;
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
+    if (w >= n_items) return;
+    const RowItem it = items[w];
+    const int row0 = __builtin_amdgcn_readfirstlane(it.row);
+    const int start = __builtin_amdgcn_readfirstlane(it.start);
+    const int end = __builtin_amdgcn_readfirstlane(it.end);
+    if (start >= end) return;
+    const int lane = lane_id();
+    const int g = lane >> 3, j = lane & 7;
+    const O rb = (O)KU * (O)sizeof(T);
+    // units of the 8 A rows
+    T a[PANEL_ROWS][UPL];
+#pragma unroll
+    for (int r = 0; r < PANEL_ROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < UPL; ++i)
+            a[r][i] = load_at<T, O>(A, (O)(row0 + r) * rb + (O)((j + i * 8) * (int)sizeof(T)));
+    const int rs0 = __builtin_amdgcn_readfirstlane(rowptr[row0]);   // the shared column list
+    const int rsj = rowptr[row0 + j];                               // this lane's output row
+    const int last = end - 1;
+    auto col_off = [&](int base) {      // byte offset of the B row of this lane's column
+        const int e = base + lane < last ? base + lane : last;
+        return (O)col[rs0 + e] * rb;
+    };
+    auto reduce_step = [&](const T (&bfs)[UPL]) {
+        float keep = 0.f;
+#pragma unroll
+        for (int r = 0; r < PANEL_ROWS; ++r) {
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) p = U::dot(a[r][i], bfs[i], p);
+            p = group_sum<8>(p);
+            keep = j == r ? p : keep;
+        }
+        return keep;
+    };
+    if constexpr (UPL == 1) {
+        // Three chunks in flight, every load unconditional (clamped) so that the wait
+        // counts stay exact: iteration i loads the column indices of chunk i+2, the B
+        // units and S values of chunk i+1, and computes chunk i.
+        auto gather = [&](O boff, T (&bf)[8][1]) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) bf[t][0] = load_at<T, O>(B, shfl_off<O>(boff, t * 8 + g) + (O)(j * (int)sizeof(T)));
+        };
+        auto load_s = [&](int base, float (&sv)[8]) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int et = base + t * 8 + g < last ? base + t * 8 + g : last;
+                sv[t] = sval[rsj + et];
+            }
+        };
+        T bf_cur[8][1], bf_nxt[8][1];
+        float sv_cur[8], sv_nxt[8];
+        O boff_nxt = col_off(start + WAVE);
+        {
+            const O boff0 = col_off(start);
+            gather(boff0, bf_cur);
+            load_s(start, sv_cur);
+        }
+        for (int base = start; base < end; base += WAVE) {
+            const O boff_nn = col_off(base + 2 * WAVE);
+            gather(boff_nxt, bf_nxt);
+            load_s(base + WAVE, sv_nxt);
+            float out[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) out[t] = reduce_step(bf_cur[t]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int et = base + t * 8 + g;
+                if (et < end) P[rsj + et] = out[t] * sv_cur[t];
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) { bf_cur[t][0] = bf_nxt[t][0]; sv_cur[t] = sv_nxt[t]; }
+            boff_nxt = boff_nn;
+        }
+    } else {
+        constexpr int NB = 8 / UPL < 1 ? 1 : 8 / UPL;               // steps per batch of gathers
+        O boff = col_off(start);
+        for (int base = start; base < end; base += WAVE) {
+            const O boff_nxt = col_off(base + WAVE);                // travels while this chunk computes
+            float sv[8], out[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int et = base + t * 8 + g < last ? base + t * 8 + g : last;
+                sv[t] = sval[rsj + et];
+            }
+#pragma unroll
+            for (int t0 = 0; t0 < 8; t0 += NB) {
+                T bf[NB][UPL];
+#pragma unroll
+                for (int s = 0; s < NB; ++s) {
+                    const O bo = shfl_off<O>(boff, (t0 + s) * 8 + g);
+#pragma unroll
+                    for (int i = 0; i < UPL; ++i) bf[s][i] = load_at<T, O>(B, bo + (O)((j + i * 8) * (int)sizeof(T)));
+                }
+#pragma unroll
+                for (int s = 0; s < NB; ++s) out[t0 + s] = reduce_step(bf[s]);
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int et = base + t * 8 + g;
+                if (et < end) P[rsj + et] = out[t] * sv[t];
+            }
+            boff = boff_nxt;
+        }
     }
 }
 

@@ -15,7 +15,8 @@ struct PlanCounters {
     unsigned long long rows_short, rows_medium, rows_long;
     unsigned long long nnz_short, nnz_medium, nnz_long;
     unsigned long long n_items;    // work items of the wave-per-segment kernel
-    unsigned long long spare[6];
+    unsigned long long n_tiles, nnz_tiles, tiles_scanned;     // dense-tile path
+    unsigned long long n_panels, nnz_panels, panel_items;     // row-panel path
 };
 
 __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
@@ -126,12 +127,12 @@ constexpr int SCAN_BLOCK = 256;
 constexpr int SCAN_ITEMS = 4;                       // rows per thread
 constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;  // rows per block
 
-// strip_ntiles (may be null): rows of a strip that the dense-tile path owns count
-// as empty here
+// owner8 (may be null): one byte per group of 8 rows, non-zero when the dense-tile
+// path (1) or the row-panel path (2) computes those rows; they count as empty here
 __device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr,
-                                                       const unsigned int *__restrict__ strip_ntiles, int64_t i,
+                                                       const unsigned char *__restrict__ owner8, int64_t i,
                                                        int M, int ts, int seg, unsigned int *len_out) {
-    if (i >= M || (strip_ntiles && strip_ntiles[i >> 4] != 0)) { *len_out = 0; return 0; }
+    if (i >= M || (owner8 && owner8[i >> 3] != 0)) { *len_out = 0; return 0; }
     const unsigned int len = (unsigned int)(rowptr[i + 1] - rowptr[i]);
     *len_out = len;
     return len >= (unsigned int)ts ? (len + seg - 1) / seg : 0u;
@@ -162,7 +163,7 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 
 // pass 1: items per block of SCAN_TILE rows, plus the row statistics
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
-                                                               const unsigned int *__restrict__ strip_ntiles, int M,
+                                                               const unsigned char *__restrict__ owner8, int M,
                                                                int ts, int seg, unsigned int *__restrict__ block_sums,
                                                                PlanCounters *pc) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        const unsigned int cnt = row_item_count(rowptr, strip_ntiles, base + q, M, ts, seg, &len);
+        const unsigned int cnt = row_item_count(rowptr, owner8, base + q, M, ts, seg, &len);
         items += cnt;
         if (len == 0) continue;
         if (cnt == 0) { ++r_short; n_short += len; }
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__
 
 // pass 3: write the items
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr,
-                                                               const unsigned int *__restrict__ strip_ntiles, int M,
+                                                               const unsigned char *__restrict__ owner8, int M,
                                                                int ts, int seg,
                                                                const unsigned int *__restrict__ block_offsets,
                                                                RowItem *__restrict__ items) {
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
     unsigned int cnt[SCAN_ITEMS], mine = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        cnt[q] = row_item_count(rowptr, strip_ntiles, base + q, M, ts, seg, &len);
+        cnt[q] = row_item_count(rowptr, owner8, base + q, M, ts, seg, &len);
         mine += cnt[q];
     }
     unsigned int total;
@@ -231,6 +232,65 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
             const int32_t b = a + seg < e ? a + seg : e;
             items[at++] = RowItem{row, a, b, 0};
         }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Row-panel detector: panel p = rows [8p, 8p+8).  It qualifies when all 8 rows
+// exist, are not owned by the dense-tile path, have the same length >= min_len and
+// the same column list.  One wavefront per panel; lanes stride over the list.
+// counts[p] = work items of the panel (ceil(len/pseg)) or 0; owner8[p] = 2 when taken.
+__global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__ rowptr,
+                                                     const int32_t *__restrict__ col, int M, int64_t n_panels,
+                                                     int min_len, int pseg, unsigned char *__restrict__ owner8,
+                                                     unsigned int *__restrict__ counts, PlanCounters *pc) {
+    const int64_t p = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (p >= n_panels) return;
+    const int lane = lane_id();
+    const int64_t row0 = p * 8;
+    bool ok = row0 + 8 <= M && owner8[p] == 0;
+    int s0 = 0, len = 0;
+    if (ok) {
+        s0 = rowptr[row0];
+        len = rowptr[row0 + 1] - s0;
+        ok = len >= min_len;
+        for (int r = 1; ok && r < 8; ++r) ok = rowptr[row0 + r + 1] - rowptr[row0 + r] == len;
+    }
+    // ok is the same in every lane here
+    if (ok) {
+        bool differ = false;
+        for (int e = lane; e < len; e += WAVE) {
+            const int c0 = col[s0 + e];
+            for (int r = 1; r < 8; ++r) differ |= col[rowptr[row0 + r] + e] != c0;
+        }
+        ok = __ballot(differ) == 0;
+    }
+    if (lane == 0) {
+        counts[p] = ok ? (unsigned int)((len + pseg - 1) / pseg) : 0u;
+        if (ok) {
+            owner8[p] = 2;
+            atomicAdd(&pc->n_panels, 1ull);
+            atomicAdd(&pc->nnz_panels, (unsigned long long)len * 8ull);
+        }
+    }
+}
+
+// items of the taken panels: {first row, [start,end) inside the shared list}
+__global__ __launch_bounds__(256) void k_panel_items(const int32_t *__restrict__ rowptr, int64_t n_panels, int pseg,
+                                                     const unsigned int *__restrict__ counts,
+                                                     const unsigned int *__restrict__ offsets,
+                                                     RowItem *__restrict__ items) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_panels) return;
+    const unsigned int n = counts[p];
+    if (n == 0) return;
+    const int32_t row0 = (int32_t)(p * 8);
+    const int32_t len = rowptr[row0 + 1] - rowptr[row0];
+    unsigned int at = offsets[p];
+    for (unsigned int k = 0; k < n; ++k) {
+        const int32_t a = (int32_t)k * pseg;
+        const int32_t b = a + pseg < len ? a + pseg : len;
+        items[at++] = RowItem{row0, a, b, 0};
     }
 }
 

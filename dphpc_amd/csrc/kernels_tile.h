@@ -92,7 +92,7 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
 __global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ rowptr,
                                                     const int32_t *__restrict__ col, int M, int64_t n_strips,
                                                     int min_fill, unsigned int *__restrict__ strip_ntiles,
-                                                    PlanCounters *pc) {
+                                                    unsigned char *__restrict__ owner8, PlanCounters *pc) {
     const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int sub = threadIdx.x & 15;
     if (strip >= n_strips) return;   // whole 16-lane rows leave together
@@ -107,8 +107,10 @@ __global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ 
     if (sub == 0) {
         strip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
         if (take) {
-            atomicAdd(&pc->spare[0], (unsigned long long)tiles);        // tiles on the MFMA path
-            atomicAdd(&pc->spare[1], (unsigned long long)all_entries);  // entries they cover
+            owner8[2 * strip] = 1;         // both 8-row halves (the array is padded to an even length)
+            owner8[2 * strip + 1] = 1;
+            atomicAdd(&pc->n_tiles, (unsigned long long)tiles);
+            atomicAdd(&pc->nnz_tiles, (unsigned long long)all_entries);
         }
     }
 }

@@ -62,7 +62,16 @@ struct sddmm_ctx {
     TileDesc *d_tiles = nullptr;
     int64_t n_tiles = 0, tiles_cap = 0, nnz_tiles = 0;
     int tile_steps = 0, tiles_per_wave = 8;
-    bool tiles_active = false;       // d_strip_ntiles describes the current pattern
+    bool tiles_active = false;       // d_tiles describes the current pattern
+    // row ownership (one byte per 8 rows: 0 rows kernels, 1 dense tiles, 2 row panels)
+    unsigned char *d_owner8 = nullptr;
+    int64_t owner_cap = 0;
+    bool owner_active = false;
+    // row-panel path
+    unsigned int *d_panel_counts = nullptr, *d_panel_off = nullptr;
+    int64_t panels_cap = 0;
+    RowItem *d_panel_items = nullptr;
+    int64_t n_panel_items = 0, panel_items_cap = 0, n_panels = 0, nnz_panels = 0;
 };
 
 namespace {
@@ -119,6 +128,13 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_strip_ntiles);
     dfree(c->d_strip_off);
     dfree(c->d_tiles);
+    dfree(c->d_owner8);
+    dfree(c->d_panel_counts);
+    dfree(c->d_panel_off);
+    dfree(c->d_panel_items);
+    c->owner_cap = c->panels_cap = c->panel_items_cap = 0;
+    c->n_panel_items = c->n_panels = c->nnz_panels = 0;
+    c->owner_active = false;
     c->items_cap = c->block_sums_cap = c->n_items = 0;
     c->strips_cap = c->tiles_cap = c->n_tiles = c->nnz_tiles = 0;
     c->tiles_active = false;
@@ -274,7 +290,7 @@ void launch_auto(sddmm_ctx *c) {
         using LT = decltype(L);
         hipLaunchKernelGGL((k_auto<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
-                           (const unsigned int *)(c->tiles_active ? c->d_strip_ntiles : nullptr), c->d_col, c->d_sval,
+                           (const unsigned char *)(c->owner_active ? c->d_owner8 : nullptr), c->d_col, c->d_sval,
                            c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
     });
 }
@@ -300,8 +316,8 @@ int classify_rows(sddmm_ctx *c) {
     c->pc = fresh;
     HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
     if (nb > 0) {
-        const unsigned int *strips = c->tiles_active ? c->d_strip_ntiles : nullptr;
-        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, strips,
+        const unsigned char *owner = c->owner_active ? c->d_owner8 : nullptr;
+        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, owner,
                            c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc);
         hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
@@ -320,20 +336,53 @@ int classify_rows(sddmm_ctx *c) {
     }
     if (c->n_items > 0) {
         hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
-                           c->tiles_active ? c->d_strip_ntiles : nullptr, c->sM, c->ts, c->seg, c->d_block_sums,
-                           c->d_items);
+                           (const unsigned char *)(c->owner_active ? c->d_owner8 : nullptr), c->sM, c->ts, c->seg,
+                           c->d_block_sums, c->d_items);
         HIP_TRY(c, hipGetLastError());
     }
     return SDDMM_OK;
 }
 
-// Dense-tile classifier.  min_fill = average stored entries per 16x16 tile a strip
-// needs to be taken.  Leaves tiles_active false when the path does not apply
-// (no row pointer, row size not a multiple of 64 bytes, nothing qualifies).
-int plan_tiles(sddmm_ctx *c, int min_fill) {
+// Exclusive scan of n unsigned ints on the device (in != out), total to *d_total.
+int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t n, unsigned long long *d_total) {
+    const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
+    if (nb > c->block_sums_cap) {
+        dfree(c->d_block_sums);
+        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
+        c->block_sums_cap = nb;
+    }
+    hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, in, n, c->d_block_sums);
+    hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb, d_total);
+    hipLaunchKernelGGL(k_scan_apply, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, in, n,
+                       (const unsigned int *)c->d_block_sums, out);
+    HIP_TRY(c, hipGetLastError());
+    return SDDMM_OK;
+}
+
+// Clears the row-ownership bytes and the tile / panel counters before the classifiers run.
+int begin_ownership(sddmm_ctx *c) {
+    const int64_t bytes = 2 * (((int64_t)c->sM + 15) / 16) + 16;
+    if (bytes > c->owner_cap) {
+        dfree(c->d_owner8);
+        ALLOC_TRY(c, c->d_owner8, (size_t)bytes);
+        c->owner_cap = bytes;
+    }
+    HIP_TRY(c, hipMemsetAsync(c->d_owner8, 0, (size_t)bytes, c->stream));
+    c->pc.n_tiles = c->pc.nnz_tiles = c->pc.tiles_scanned = 0;
+    c->pc.n_panels = c->pc.nnz_panels = c->pc.panel_items = 0;
+    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
+    c->owner_active = true;
     c->tiles_active = false;
     c->n_tiles = c->nnz_tiles = 0;
-    if (!c->have_rowptr || c->nnz == 0) return SDDMM_OK;
+    c->n_panel_items = c->n_panels = c->nnz_panels = 0;
+    return SDDMM_OK;
+}
+
+// Dense-tile classifier.  min_fill = average stored entries per 16x16 tile a strip
+// needs to be taken.  Leaves tiles_active false when the path does not apply
+// (row size not a multiple of 64 bytes, nothing qualifies).
+int plan_tiles(sddmm_ctx *c, int min_fill) {
+    if (c->nnz == 0) return SDDMM_OK;
     const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
     if (row_bytes % 64) return SDDMM_OK;
     const int steps = (int)(row_bytes / 64);
@@ -347,29 +396,18 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
         ALLOC_TRY(c, c->d_strip_off, (size_t)n_strips * sizeof(unsigned int));
         c->strips_cap = n_strips;
     }
-    const int64_t nb = (n_strips + SCAN_TILE - 1) / SCAN_TILE;
-    if (nb > c->block_sums_cap) {
-        dfree(c->d_block_sums);
-        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
-        c->block_sums_cap = nb;
-    }
-    c->pc.spare[0] = c->pc.spare[1] = c->pc.spare[2] = 0;
-    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
     const unsigned walk_grid = (unsigned)((n_strips * 16 + 255) / 256);
     hipLaunchKernelGGL(k_tile_count, dim3(walk_grid), dim3(256), 0, c->stream, c->d_rowptr, c->d_col, c->sM, n_strips,
-                       min_fill, c->d_strip_ntiles, c->d_pc);
-    hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_strip_ntiles, n_strips,
-                       c->d_block_sums);
-    hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
-                       &c->d_pc->spare[2]);
-    hipLaunchKernelGGL(k_scan_apply, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_strip_ntiles, n_strips,
-                       c->d_block_sums, c->d_strip_off);
+                       min_fill, c->d_strip_ntiles, c->d_owner8, c->d_pc);
     HIP_TRY(c, hipGetLastError());
-    int rc = fetch_counters(c);
+    int rc = device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
     if (rc) return rc;
-    c->n_tiles = (int64_t)c->pc.spare[0];
-    c->nnz_tiles = (int64_t)c->pc.spare[1];
-    if ((int64_t)c->pc.spare[2] != c->n_tiles) return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
+    rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_tiles = (int64_t)c->pc.n_tiles;
+    c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
+    if ((int64_t)c->pc.tiles_scanned != c->n_tiles)
+        return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
     if (c->n_tiles == 0) return SDDMM_OK;
     if (c->n_tiles > c->tiles_cap) {
         dfree(c->d_tiles);
@@ -382,6 +420,69 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
     c->tiles_active = true;
     c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 8));
     return SDDMM_OK;
+}
+
+// Row-panel detector (8 consecutive rows, 8-aligned, same column list).  Applies to
+// the 8-lanes-per-entry layouts with no masked unit and 32-bit offsets.
+bool panels_applicable(const sddmm_ctx *c) {
+    const Shape s = shape_of(c);
+    // the 8 A rows of a panel live in registers (8 x UPL x 4 VGPRs per lane, plus the
+    // converted halves for bf16): K = 32 or 64 in fp32, K = 64 in bf16
+    if (s.unit == 1 || s.LPN != 8 || !s.fullk || s.wide) return false;
+    return s.unit == 0 ? s.UPL <= 2 : s.UPL == 1;
+}
+
+int plan_panels(sddmm_ctx *c, int min_len, int pseg) {
+    if (c->nnz == 0 || !panels_applicable(c)) return SDDMM_OK;
+    const int64_t n_panels = (int64_t)c->sM / 8;
+    if (n_panels == 0) return SDDMM_OK;
+    if (n_panels > c->panels_cap) {
+        dfree(c->d_panel_counts);
+        dfree(c->d_panel_off);
+        ALLOC_TRY(c, c->d_panel_counts, (size_t)n_panels * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_panel_off, (size_t)n_panels * sizeof(unsigned int));
+        c->panels_cap = n_panels;
+    }
+    hipLaunchKernelGGL(k_panel_flags, dim3((unsigned)((n_panels * WAVE + 255) / 256)), dim3(256), 0, c->stream,
+                       c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner8, c->d_panel_counts, c->d_pc);
+    HIP_TRY(c, hipGetLastError());
+    int rc = device_scan(c, c->d_panel_counts, c->d_panel_off, n_panels, &c->d_pc->panel_items);
+    if (rc) return rc;
+    rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_panels = (int64_t)c->pc.n_panels;
+    c->nnz_panels = (int64_t)c->pc.nnz_panels;
+    c->n_panel_items = (int64_t)c->pc.panel_items;
+    if (c->n_panel_items == 0) return SDDMM_OK;
+    if (c->n_panel_items > c->panel_items_cap) {
+        dfree(c->d_panel_items);
+        ALLOC_TRY(c, c->d_panel_items, (size_t)c->n_panel_items * sizeof(RowItem));
+        c->panel_items_cap = c->n_panel_items;
+    }
+    hipLaunchKernelGGL(k_panel_items, dim3((unsigned)((n_panels + 255) / 256)), dim3(256), 0, c->stream, c->d_rowptr,
+                       n_panels, pseg, (const unsigned int *)c->d_panel_counts, (const unsigned int *)c->d_panel_off,
+                       c->d_panel_items);
+    HIP_TRY(c, hipGetLastError());
+    return SDDMM_OK;
+}
+
+template <class U, int UPL>
+void launch_panel_t(sddmm_ctx *c, int KU) {
+    using LT = Layout<U, 8, UPL, true, false>;
+    const int64_t nblocks = (c->n_panel_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    hipLaunchKernelGGL((k_panel<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                       (const void *)c->dA, (const void *)c->dB, KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
+                       (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
+}
+template <class U>
+void launch_panel_u(sddmm_ctx *c, const Shape &s) {
+    if (s.UPL == 1) launch_panel_t<U, 1>(c, s.KU);
+    else launch_panel_t<U, 2>(c, s.KU);
+}
+void launch_panels(sddmm_ctx *c) {
+    const Shape s = shape_of(c);
+    if (s.unit == 0) launch_panel_u<UnitF32x4>(c, s);
+    else launch_panel_t<UnitBF16x8, 1>(c, s.KU);
 }
 
 template <bool BF16, int STEPS>
@@ -454,8 +555,10 @@ int enqueue_run(sddmm_ctx *c) {
     switch (c->strategy) {
         case SDDMM_AUTO:
         case SDDMM_MFMA_TILE:
+        case SDDMM_LDS_TILED:
             c->launches = 0;
             if (c->tiles_active && c->n_tiles > 0) { launch_tiles(c); ++c->launches; }
+            if (c->n_panel_items > 0) { launch_panels(c); ++c->launches; }
             if (c->rows_short > 0 || c->n_items > 0) { launch_auto(c); ++c->launches; }
             break;
         case SDDMM_FLAT: launch_flat(c); break;
@@ -485,12 +588,24 @@ int do_plan(sddmm_ctx *c, int strategy) {
     if (strategy == SDDMM_AUTO && !csr_ok) resolved = SDDMM_FLAT;
     switch (resolved) {
         case SDDMM_AUTO:
-        case SDDMM_MFMA_TILE: {
-            // strips first (they take whole rows away from the row classes), then rows;
-            // MFMA_TILE takes every sorted strip, AUTO only the well-filled ones
+        case SDDMM_MFMA_TILE:
+        case SDDMM_LDS_TILED: {
+            // Row ownership in this order: well-filled 16-row strips go to the MFMA tile
+            // path, then 8-row panels with a common column list to the panel kernel, the
+            // rest is split by length.  MFMA_TILE takes every sorted strip and no panel,
+            // LDS_TILED every panel and no strip; AUTO applies the thresholds.
             if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
-            int rc = plan_tiles(c, resolved == SDDMM_MFMA_TILE ? 1 : std::max(1, env_int("SDDMM_TILE_FILL", 32)));
+            int rc = begin_ownership(c);
             if (rc) return rc;
+            if (resolved != SDDMM_LDS_TILED) {
+                rc = plan_tiles(c, resolved == SDDMM_MFMA_TILE ? 1 : std::max(1, env_int("SDDMM_TILE_FILL", 96)));
+                if (rc) return rc;
+            }
+            if (resolved != SDDMM_MFMA_TILE) {
+                rc = plan_panels(c, resolved == SDDMM_LDS_TILED ? 1 : std::max(1, env_int("SDDMM_PANEL_MIN", 16)),
+                                 std::max(WAVE, env_int("SDDMM_PANEL_SEG", 512)));
+                if (rc) return rc;
+            }
             c->ts = std::max(1, env_int("SDDMM_TS", 24));
             c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
             rc = classify_rows(c);
@@ -507,8 +622,6 @@ int do_plan(sddmm_ctx *c, int strategy) {
         case SDDMM_SHORT_ROWS:
             if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
             break;
-        case SDDMM_LDS_TILED:
-            return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d is not available in this build", resolved);
         default: return fail(c, SDDMM_ERR_INVALID, "unknown strategy %d", strategy);
     }
     c->requested = strategy;
@@ -522,9 +635,11 @@ void fill_model(sddmm_ctx *c) {
     s.strategy_used = c->strategy;
     s.nnz = c->nnz;
     s.rows_nonempty = (int64_t)c->pc.rows_nonempty;
-    if (c->strategy == SDDMM_AUTO || c->strategy == SDDMM_MFMA_TILE) {
+    if (c->strategy == SDDMM_AUTO || c->strategy == SDDMM_MFMA_TILE || c->strategy == SDDMM_LDS_TILED) {
         s.mfma_tiles = c->tiles_active ? c->n_tiles : 0;
         s.nnz_mfma = c->tiles_active ? c->nnz_tiles : 0;
+        s.panels = c->n_panels;
+        s.nnz_panel = c->nnz_panels;
         s.rows_short = (int64_t)c->pc.rows_short; s.rows_medium = (int64_t)c->pc.rows_medium;
         s.rows_long = (int64_t)c->pc.rows_long;
         s.nnz_short = (int64_t)c->pc.nnz_short; s.nnz_medium = (int64_t)c->pc.nnz_medium;

@@ -62,9 +62,11 @@ enum sddmm_strategy {
                              (the role of src/competitors/gpu/gpu_convert.cu:8-50)    */
     SDDMM_ROW_WAVE = 2,   /* one wavefront per row segment, A row held in registers   */
     SDDMM_SHORT_ROWS = 3, /* many short rows per wavefront                            */
-    SDDMM_LDS_TILED = 4,  /* row panel stages its active B rows in LDS
-                             (the role of src/competitors/gpu/gpu_shared.cu:18-88 and
-                              gpu_preprocessing.cu:18-96)                             */
+    SDDMM_LDS_TILED = 4,  /* row panels: 8 rows with a common column list share every
+                             gathered B row, A rows held in registers; other rows on
+                             AUTO's gather kernels (the role of the row-panel kernels
+                             src/competitors/gpu/gpu_shared.cu:18-88 and
+                             gpu_preprocessing.cu:18-96: B reused across a row panel) */
     SDDMM_MFMA_TILE = 5,  /* near-dense 16x16 tiles on MFMA, remainder on AUTO's
                              gather kernels (the role of gpu_tensor.cu:27-99)         */
     SDDMM_EXACT = 6       /* one lane per entry, k ascending, separate fp32 multiply
@@ -92,6 +94,8 @@ typedef struct sddmm_stats {
        gathered = 4(M+1) + 12 nnz + e K rows_nonempty + e K nnz  (e = 4 or 2)         */
     double flops;
     double bytes_gathered;
+    int64_t panels;           /* 8-row panels with a common column list (panel kernel) */
+    int64_t nnz_panel;        /* stored entries covered by those panels               */
 } sddmm_stats;
 
 /* ---- life cycle --------------------------------------------------------- */

@@ -19,7 +19,7 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 f32 = np.float32
 
-FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.MFMA_TILE, capi.EXACT]
+FP32_STRATEGIES = [capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.LDS_TILED, capi.MFMA_TILE, capi.EXACT]
 
 
 def _say(*a):
@@ -390,14 +390,15 @@ def test_tiles_partial_fill_ragged_edges_and_mixed_strips(engine_factory):
         got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, strategy)
         assert_parity(got, rowptr, col, val, A, B, what="mixed strips")
         assert st.mfma_tiles > 0 and 0 < st.nnz_mfma < len(col)
-        assert st.kernels_launched == 2
+        assert st.kernels_launched >= 2
     rows = np.repeat(np.arange(M), np.diff(rowptr))
     forced = rows // 16 != 4                                   # MFMA_TILE: every strip but the unsorted one
     assert st.nnz_mfma == np.count_nonzero(forced)
     assert st.mfma_tiles == _tile_count(rowptr, col, M) - len(np.unique(col[rows // 16 == 4] // 16))
-    # AUTO leaves the sparse strip to the gather kernels as well
+    # AUTO takes only the strips whose tiles are well filled
     _, st_auto = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.AUTO)
-    assert st_auto.nnz_mfma == np.count_nonzero(forced & (rows // 16 != 3))
+    assert 0 < st_auto.nnz_mfma < st.nnz_mfma
+    assert st_auto.nnz_mfma >= np.count_nonzero(rows // 16 == 0)
 
 
 def test_tile_path_not_applicable_falls_back_to_gather(engine_factory):
@@ -409,8 +410,74 @@ def test_tile_path_not_applicable_falls_back_to_gather(engine_factory):
     assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B)
 
 
-def test_fem_blocks_take_the_tile_path(engine_factory):
+def test_fem_blocks_tiles_and_panels(engine_factory):
     w = W.make("fem_banded", "small")
-    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.MFMA_TILE)
     assert st.nnz_mfma == w.nnz and st.mfma_tiles == _tile_count(w.rowptr, w.col, w.M)
     assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem tiles")
+    # every block row is an 8-row panel with one column list
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.LDS_TILED)
+    assert st.panels == w.M // 8 and st.nnz_panel == w.nnz and st.mfma_tiles == 0
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem panels")
+    flat, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.FLAT)
+    np.testing.assert_array_equal(got.view(np.uint32), flat.view(np.uint32))   # same per-entry arithmetic
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
+    assert st.nnz_mfma + st.nnz_panel == w.nnz
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem auto")
+
+
+@pytest.mark.parametrize("K,dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (64, "bf16"), (256, "bf16"),
+                                     (24, "f32"), (33, "f32")])
+def test_row_panels(engine_factory, K, dtype):
+    """Groups of identical rows: aligned 8-row panels are taken, everything else
+    (unaligned groups, groups of other sizes, rows with one differing column, short
+    lists, the ragged tail) stays on the row kernels."""
+    rng = np.random.default_rng(100 + K)
+    N = 700
+    rows_cols = []
+
+    def add_group(n_rows, length):
+        cols = np.sort(rng.choice(N, length, replace=False))
+        for _ in range(n_rows):
+            rows_cols.append(cols.copy())
+
+    add_group(8, 300)          # rows 0-7    panel, several segments
+    add_group(8, 70)           # rows 8-15   panel
+    add_group(3, 40)           # rows 16-18  too few rows ...
+    add_group(8, 40)           # rows 19-26  ... and this group is not 8-aligned
+    add_group(5, 0)            # rows 27-31  empty rows
+    add_group(16, 33)          # rows 32-47  two panels
+    add_group(8, 50)           # rows 48-55  one row differs in one column below
+    add_group(8, 9)            # rows 56-63  shorter than AUTO's minimum (still a panel for LDS_TILED)
+    add_group(5, 20)           # rows 64-68  ragged tail
+    c = rows_cols[51].copy()
+    c[7] = np.setdiff1d(np.arange(N), c)[5]                # a column the group does not have
+    rows_cols[51] = np.sort(c)
+    M = len(rows_cols)
+    lens = np.array([len(x) for x in rows_cols])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows_cols).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == "bf16":
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K)
+        ops, dt = (Ab, Bb), capi.BF16
+    else:
+        ops, dt = (A, B), capi.F32
+    applicable = (dtype, K) in (("f32", 32), ("f32", 64), ("bf16", 64))     # A rows of a panel fit in registers
+    same = len(rows_cols[51]) == 50 and np.array_equal(rows_cols[51], rows_cols[48])
+    assert not same
+    for strategy, min_len in ((capi.LDS_TILED, 1), (capi.AUTO, 16)):
+        _say("panels", K, dtype, capi.STRATEGY_NAMES[strategy])
+        got, st = run_csr(engine_factory, rowptr, col, val, *ops, N, strategy, dt)
+        assert_parity(got, rowptr, col, val, A, B, what="panels K=%d" % K)
+        if strategy == capi.LDS_TILED:
+            exp = [(0, 300), (8, 70), (32, 33), (40, 33), (56, 9)] if applicable else []
+            assert st.panels == len(exp) and st.nnz_panel == sum(8 * l for _, l in exp)
+            assert st.mfma_tiles == 0
+    if applicable:
+        flat, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.FLAT, dt)
+        lds, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.LDS_TILED, dt)
+        np.testing.assert_array_equal(flat.view(np.uint32), lds.view(np.uint32))
