@@ -57,7 +57,8 @@ __device__ __forceinline__ int sum16(int v) {
 
 // Walks the tiles of one strip in increasing tile column.  All 16 lanes of the
 // strip call on_tile(tj, first, mask) together; `first` / `mask` are this lane's
-// row's first position and column mask in the tile (mask 0: row absent).
+// row's first position and column mask in the tile (mask 0: row absent).  The walk
+// stops early when on_tile returns false (it must return the same in all 16 lanes).
 // Returns false in a lane whose row is not strictly increasing in column.
 template <class F>
 __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M,
@@ -81,7 +82,7 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
             ++p;
             c = p < end ? col[p] : -1;
         }
-        on_tile(t, first, mask);
+        if (!on_tile(t, first, mask)) break;
     }
     return sorted;
 }
@@ -96,14 +97,21 @@ __global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ 
     const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int sub = threadIdx.x & 15;
     if (strip >= n_strips) return;   // whole 16-lane rows leave together
+    // entries of the strip, known from rowptr alone: the walk can stop as soon as the
+    // strip has more tiles than that many entries could fill to the threshold
+    const int64_t r_lo = strip * 16, r_hi = r_lo + 16 < M ? r_lo + 16 : M;
+    const int64_t strip_entries = (int64_t)rowptr[r_hi] - (int64_t)rowptr[r_lo];
+    const int64_t max_tiles = strip_entries / min_fill;
     int tiles = 0, entries = 0;
     const bool sorted = walk_strip(rowptr, col, M, strip, sub, [&](int, int, unsigned int mask) {
         ++tiles;
         entries += __builtin_popcount(mask);
+        return (int64_t)tiles <= max_tiles;
     });
     const int all_entries = sum16(entries);
     const int unsorted = sum16(sorted ? 0 : 1);
-    const bool take = unsorted == 0 && tiles > 0 && (int64_t)all_entries >= (int64_t)min_fill * tiles;
+    const bool take = unsorted == 0 && tiles > 0 && (int64_t)tiles <= max_tiles &&
+                      (int64_t)all_entries >= (int64_t)min_fill * tiles;
     if (sub == 0) {
         strip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
         if (take) {
@@ -132,6 +140,7 @@ __global__ __launch_bounds__(256) void k_tile_fill(const int32_t *__restrict__ r
         d->mask[sub] = (uint16_t)mask;
         if (sub == 0) { d->strip = (int32_t)strip; d->tj = tj; d->pad[0] = 0; d->pad[1] = 0; }
         ++at;
+        return true;
     });
 }
 
