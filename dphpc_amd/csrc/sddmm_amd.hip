@@ -610,6 +610,17 @@ int do_plan(sddmm_ctx *c, int strategy) {
             c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
             rc = classify_rows(c);
             if (rc) return rc;
+            // A matrix whose rows are short on average (fewer than 32 entries per non-empty
+            // row), with no strip or panel taken, is a flat stream of entries: the flat
+            // kernel (row index per entry, perfectly balanced) measured 6 % faster there than
+            // the row split (power-law shape, K=32: 634 us against 672 us).
+            const double avg_len = c->pc.rows_nonempty ? (double)c->nnz / (double)c->pc.rows_nonempty : 0.0;
+            if (resolved == SDDMM_AUTO && c->n_tiles == 0 && c->n_panel_items == 0 &&
+                avg_len < (double)env_int("SDDMM_FLAT_AVG", 32)) {
+                rc = ensure_rowidx(c);
+                if (rc) return rc;
+                resolved = SDDMM_FLAT;
+            }
             break;
         }
         case SDDMM_FLAT:

@@ -78,8 +78,10 @@ enum sddmm_strategy {
 typedef struct sddmm_stats {
     float plan_ms;            /* classifier + auxiliary structure build               */
     float run_ms;             /* all kernels of the last sddmm_run                    */
-    int32_t strategy_used;    /* SDDMM_AUTO = per-row dispatch; a fixed strategy
-                                 otherwise (also when AUTO had to fall back to one)   */
+    int32_t strategy_used;    /* SDDMM_AUTO = per-strip/panel/row dispatch; a fixed
+                                 strategy otherwise -- also when AUTO resolved to one
+                                 (FLAT for unsorted COO and for matrices whose rows
+                                 are short on average)                                */
     int32_t kernels_launched; /* launches per sddmm_run                               */
     int64_t nnz;
     int64_t rows_nonempty;

@@ -1,0 +1,118 @@
+"""Device-resident operands (the *_device entry points) and operands of 4 GiB and
+more (64-bit byte offsets in the gather kernels).  HIP memory is managed here with
+a few direct runtime calls; the library only borrows the pointers."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from dphpc_amd import capi
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+class Hip:
+    def __init__(self):
+        self.h = C.CDLL("libamdhip64.so")
+        self.h.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        self.h.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        self.h.hipFree.argtypes = [C.c_void_p]
+        self.live = []
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a)
+        p = C.c_void_p()
+        assert self.h.hipMalloc(C.byref(p), max(a.nbytes, 16)) == 0
+        assert self.h.hipMemcpy(p, a.ctypes.data_as(C.c_void_p), a.nbytes, 1) == 0     # host to device
+        self.live.append(p)
+        return p
+
+    def download(self, p, n, dtype):
+        out = np.empty(n, dtype)
+        assert self.h.hipMemcpy(out.ctypes.data_as(C.c_void_p), p, out.nbytes, 2) == 0  # device to host
+        return out
+
+    def free_all(self):
+        for p in self.live:
+            self.h.hipFree(p)
+        self.live = []
+
+
+def test_device_resident_operands(engine_factory):
+    rng = np.random.default_rng(50)
+    M, N, K = 300, 260, 32
+    mask = rng.random((M, N)) < 0.1
+    r, c = np.nonzero(mask)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    ref = O.sddmm_csr(rowptr, col, val, A, B)
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    hip = Hip()
+    e = engine_factory()            # creates the context (and selects the device) first
+    try:
+        dA, dB = hip.upload(A), hip.upload(B)
+        d_rp, d_col, d_val = hip.upload(rowptr), hip.upload(col), hip.upload(val)
+        L = e.L
+        e._chk(L.sddmm_set_dense_device(e.h, M, N, K, dA, dB, capi.F32))
+        e._chk(L.sddmm_set_csr_device(e.h, M, N, len(col), d_rp, d_col, d_val))
+        e.nnz = len(col)
+        for strategy in (capi.AUTO, capi.ROW_WAVE, capi.FLAT, capi.EXACT, capi.MFMA_TILE):
+            e.plan(strategy)
+            e.run()
+            got = e.values()
+            assert O.check_values(got, ref, mag=mag)[0], capi.STRATEGY_NAMES[strategy]
+            dP = C.c_void_p()
+            e._chk(L.sddmm_get_values_device(e.h, C.byref(dP)))
+            np.testing.assert_array_equal(hip.download(dP, len(col), f32), got)
+        # borrowed values cannot be replaced through the context
+        with pytest.raises(capi.SddmmError) as ei:
+            e.update_values(val)
+        assert ei.value.code == capi.ERR_STATE
+        # a malformed device CSR is rejected by the device-side validation
+        bad = col.copy()
+        bad[5] = N
+        d_bad = hip.upload(bad)
+        assert L.sddmm_set_csr_device(e.h, M, N, len(col), d_rp, d_bad, d_val) == capi.ERR_PATTERN
+        # misaligned dense pointers are refused
+        assert L.sddmm_set_dense_device(e.h, M - 1, N, K, C.c_void_p(dA.value + 4), dB, capi.F32) == capi.ERR_INVALID
+    finally:
+        e.close()                   # the context goes first, the borrowed buffers after it
+        hip.free_all()
+
+
+def test_operand_beyond_4gib_uses_64bit_offsets(engine_factory):
+    """B of 4 GiB + a little: rows near the end sit beyond a 32-bit byte offset."""
+    K = 32
+    N = (1 << 25) + 64                       # N*K*4 bytes = 4 GiB + 8 KiB
+    M = 64
+    print("allocating %.2f GiB for B" % (N * K * 4 / 2 ** 30), flush=True)
+    sys.stdout.flush()
+    rng = np.random.default_rng(51)
+    B = np.zeros((N, K), f32)
+    hot = np.unique(np.concatenate([np.arange(0, 40), np.arange(N - 90, N), rng.integers(0, N, 300),
+                                    (1 << 25) + np.arange(-20, 20), (1 << 24) + np.arange(-5, 5)]))
+    B[hot] = rng.uniform(-1, 1, (len(hot), K)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    rows_cols = [np.sort(rng.choice(hot, size=int(rng.integers(1, 120)), replace=False)) for _ in range(M)]
+    lens = np.array([len(x) for x in rows_cols])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows_cols).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    ref = O.sddmm_csr(rowptr, col, val, A, B)
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    assert np.count_nonzero(ref) > 0.9 * len(ref)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    for strategy in (capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.LDS_TILED, capi.MFMA_TILE, capi.EXACT):
+        e.plan(strategy)
+        e.run()
+        got = e.values()
+        ok, worst, i = O.check_values(got, ref, mag=mag)
+        assert ok, (capi.STRATEGY_NAMES[strategy], i, got[i], ref[i])
+    e.close()

@@ -304,9 +304,19 @@ def test_bf16_inputs_gather_path(engine_factory, K):
         assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, rtol=1e-5, exact=(strategy == capi.EXACT), what="bf16")
 
 
-def test_auto_row_classes_and_segments(engine_factory):
+def test_auto_resolves_to_flat_when_short_rows_dominate(engine_factory):
+    w = W.make("power_law", "small")
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
+    assert st.strategy_used == capi.FLAT
+    flat, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.FLAT)
+    np.testing.assert_array_equal(got.view(np.uint32), flat.view(np.uint32))
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B)
+
+
+def test_auto_row_classes_and_segments(engine_factory, monkeypatch):
     """AUTO: rows below the short threshold go to the many-rows kernel, the rest to
     wave-per-segment items; very long rows are cut into several segments."""
+    monkeypatch.setenv("SDDMM_FLAT_AVG", "0")            # keep the row split whatever the average row length
     rng = np.random.default_rng(21)
     M, N, K = 1000, 6000, 32
     lens = rng.integers(0, 20, M)
