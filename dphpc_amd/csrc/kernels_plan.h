@@ -285,12 +285,16 @@ __global__ __launch_bounds__(256) void k_panel_items(const int32_t *__restrict__
     const unsigned int n = counts[p];
     if (n == 0) return;
     const int32_t row0 = (int32_t)(p * 8);
-    const int32_t len = rowptr[row0 + 1] - rowptr[row0];
+    const int32_t rs0 = rowptr[row0];
+    const int32_t len = rowptr[row0 + 1] - rs0;
     unsigned int at = offsets[p];
     for (unsigned int k = 0; k < n; ++k) {
         const int32_t a = (int32_t)k * pseg;
         const int32_t b = a + pseg < len ? a + pseg : len;
-        items[at++] = RowItem{row0, a, b, 0};
+        // pad carries the CSR position of the panel's first row: the 8 rows have the same
+        // length and follow each other, so row r starts at pad + r*len and a kernel can
+        // start reading the column list without first waiting for a row pointer
+        items[at++] = RowItem{row0, a, b, rs0};
     }
 }
 

@@ -294,4 +294,131 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
     }
 }
 
+// ---------------------------------------------------------------------------
+// ROW PANEL on the matrix cores: 8 consecutive rows with one column list (see
+// k_panel_flags).  One wavefront per work item = entries [start,end) of the shared
+// list, 16 columns per MFMA accumulator:
+//
+//     D[c][r] = sum_k B[col_c][k] * A[row0+r][k]      c = 0..15, r = 0..7 (8..15 unused)
+//
+// The 16 gathered B rows are the "row" operand (lane l: B row of column l&15,
+// 16-byte unit 4s + (l>>4) in step s), the 8 A rows of the panel the "column"
+// operand, held in registers for the whole item.  Result register i of lane l is
+// D[4*(l>>4)+i][l&15]: four CONSECUTIVE entries of row (l&15), so S values and P
+// move as one 16-byte access per lane (rows start at arbitrary 4-byte offsets;
+// global 16-byte accesses need no more alignment than that).  The column indices
+// are read once for the 8 rows, each gathered B unit serves 8 rows.
+// Pipeline: the entries are walked in chunks of 64 = 4 groups of 16 columns.  While
+// chunk c computes, the B units and S values of chunk c+1 are in flight (a group is
+// re-requested as soon as its registers have been consumed) and the column indices
+// of chunk c+2 are being read; every load is unconditional (clamped), so the wait
+// counts stay exact and a group only ever waits for loads issued four groups earlier.
+struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
+
+template <bool BF16, int STEPS>
+__global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+                                                      const int32_t *__restrict__ rowptr,
+                                                      const int32_t *__restrict__ col,
+                                                      const float *__restrict__ sval, float *__restrict__ P,
+                                                      const RowItem *__restrict__ items, int64_t n_items,
+                                                      int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
+    if (w >= n_items) return;
+    const RowItem it = items[w];
+    const int row0 = __builtin_amdgcn_readfirstlane(it.row);
+    const int start = __builtin_amdgcn_readfirstlane(it.start);
+    const int end = __builtin_amdgcn_readfirstlane(it.end);
+    if (start >= end) return;
+    const int lane = lane_id();
+    const int n = lane & 15, q = lane >> 4;
+    constexpr int ROW_UNITS = STEPS * 4;
+    constexpr int GROUPS = 4;                                   // groups of 16 columns per chunk
+    const uint4 *__restrict__ Au = (const uint4 *)A;
+    const uint4 *__restrict__ Bu = (const uint4 *)B;
+    // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored
+    uint4 a[STEPS];
+    {
+        const uint4 *src = Au + (int64_t)(row0 + (n & 7)) * ROW_UNITS + q;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
+    }
+    // the 8 rows of a panel have one length and follow each other in the CSR arrays
+    const int rs0 = __builtin_amdgcn_readfirstlane(it.pad);
+    const int row_len = __builtin_amdgcn_readfirstlane(rowptr[row0 + 1]) - rs0;
+    const int64_t out_row = (int64_t)rs0 + (int64_t)(n & 7) * row_len;   // this lane's output row starts here
+    const int last = end - 1;
+    auto cols_of_chunk = [&](int base) {                        // column of entry base + lane (clamped)
+        const int e = base + lane < last ? base + lane : last;
+        return col[rs0 + e];
+    };
+    struct Oper {
+        uint4 b[STEPS];
+        F4u s;
+    };
+    auto load_oper = [&](int c, int g0) {
+        Oper o;
+        const uint4 *src = Bu + (int64_t)c * ROW_UNITS + q;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
+        // S values of entries g0+4q .. g0+4q+3 of this lane's row.  The window is clamped
+        // into the row (rows of a panel hold at least 4 entries); a clamped window is
+        // only ever read for the tail group, which fetches its S values again.
+        const int e = g0 + 4 * q < row_len - 4 ? g0 + 4 * q : row_len - 4;
+        o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
+        return o;
+    };
+    auto compute_store = [&](const Oper &o, int g0) {
+        if (g0 >= end) return;                                   // wave-uniform
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            if constexpr (BF16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, o.b[s]),
+                                                              __builtin_bit_cast(bf16x8_t, a[s]), acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].x),
+                                                           __builtin_bit_cast(float, a[s].x), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].y),
+                                                           __builtin_bit_cast(float, a[s].y), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].z),
+                                                           __builtin_bit_cast(float, a[s].z), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].w),
+                                                           __builtin_bit_cast(float, a[s].w), acc, 0, 0, 0);
+            }
+        }
+        if (n < 8) {
+            const int e = g0 + 4 * q;
+            if (g0 + 16 <= end) {
+                // full group: four consecutive entries per lane
+                F4u out{acc[0] * o.s.x, acc[1] * o.s.y, acc[2] * o.s.z, acc[3] * o.s.w};
+                *reinterpret_cast<F4u *>(P + out_row + e) = out;
+            } else {
+                // tail group: the S values were read from a clamped window, fetch them again
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (e + i < end) P[out_row + e + i] = acc[i] * sval[out_row + e + i];
+            }
+        }
+    };
+
+    Oper o[GROUPS];
+    {
+        const int cc0 = cols_of_chunk(start);
+#pragma unroll
+        for (int u = 0; u < GROUPS; ++u) o[u] = load_oper(__shfl(cc0, u * 16 + n, WAVE), start + 16 * u);
+    }
+    int cc_nxt = cols_of_chunk(start + WAVE);                   // columns of the next chunk
+    for (int base = start; base < end; base += WAVE) {
+        const int cc_nn = cols_of_chunk(base + 2 * WAVE);
+#pragma unroll
+        for (int u = 0; u < GROUPS; ++u) {
+            compute_store(o[u], base + 16 * u);
+            o[u] = load_oper(__shfl(cc_nxt, u * 16 + n, WAVE), base + WAVE + 16 * u);
+        }
+        cc_nxt = cc_nn;
+    }
+}
+
 }  // namespace sddmm

@@ -72,6 +72,7 @@ struct sddmm_ctx {
     int64_t panels_cap = 0;
     RowItem *d_panel_items = nullptr;
     int64_t n_panel_items = 0, panel_items_cap = 0, n_panels = 0, nnz_panels = 0;
+    bool panel_mfma = false;         // panels run on k_panel_mfma (else on k_panel)
 };
 
 namespace {
@@ -422,18 +423,28 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
     return SDDMM_OK;
 }
 
-// Row-panel detector (8 consecutive rows, 8-aligned, same column list).  Applies to
-// the 8-lanes-per-entry layouts with no masked unit and 32-bit offsets.
-bool panels_applicable(const sddmm_ctx *c) {
+// Row-panel detector (8 consecutive rows, 8-aligned, same column list).  Two
+// kernels can run the panels: the MFMA one (row size a multiple of 64 bytes, up to
+// 1 KiB) and the VALU one (8-lanes-per-entry layouts whose 8 A rows fit in
+// registers: fp32 K = 32 or 64, bf16 K = 64, 32-bit offsets); the VALU kernel has
+// the per-entry arithmetic of the gather kernels, the MFMA kernel is faster.
+int panel_mfma_steps(const sddmm_ctx *c) {
+    const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
+    if (row_bytes % 64) return 0;
+    const int steps = (int)(row_bytes / 64);
+    return (steps == 1 || steps == 2 || steps == 4 || steps == 8 || steps == 16) ? steps : 0;
+}
+bool panel_valu_applicable(const sddmm_ctx *c) {
     const Shape s = shape_of(c);
-    // the 8 A rows of a panel live in registers (8 x UPL x 4 VGPRs per lane, plus the
-    // converted halves for bf16): K = 32 or 64 in fp32, K = 64 in bf16
     if (s.unit == 1 || s.LPN != 8 || !s.fullk || s.wide) return false;
     return s.unit == 0 ? s.UPL <= 2 : s.UPL == 1;
 }
 
 int plan_panels(sddmm_ctx *c, int min_len, int pseg) {
-    if (c->nnz == 0 || !panels_applicable(c)) return SDDMM_OK;
+    if (c->nnz == 0) return SDDMM_OK;
+    c->panel_mfma = panel_mfma_steps(c) != 0 && env_int("SDDMM_PANEL_MFMA", 1) != 0;
+    if (!c->panel_mfma && !panel_valu_applicable(c)) return SDDMM_OK;
+    if (c->panel_mfma) min_len = std::max(min_len, 4);   // 16-byte S/P accesses stay inside a row
     const int64_t n_panels = (int64_t)c->sM / 8;
     if (n_panels == 0) return SDDMM_OK;
     if (n_panels > c->panels_cap) {
@@ -479,7 +490,30 @@ void launch_panel_u(sddmm_ctx *c, const Shape &s) {
     if (s.UPL == 1) launch_panel_t<U, 1>(c, s.KU);
     else launch_panel_t<U, 2>(c, s.KU);
 }
+template <bool BF16, int STEPS>
+void launch_panel_mfma_t(sddmm_ctx *c) {
+    const int64_t nblocks = (c->n_panel_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    hipLaunchKernelGGL((k_panel_mfma<BF16, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                       (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
+                       c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
+}
+template <bool BF16>
+void launch_panel_mfma_steps(sddmm_ctx *c) {
+    switch (panel_mfma_steps(c)) {
+        case 1: launch_panel_mfma_t<BF16, 1>(c); break;
+        case 2: launch_panel_mfma_t<BF16, 2>(c); break;
+        case 4: launch_panel_mfma_t<BF16, 4>(c); break;
+        case 8: launch_panel_mfma_t<BF16, 8>(c); break;
+        default: launch_panel_mfma_t<BF16, 16>(c); break;
+    }
+}
+
 void launch_panels(sddmm_ctx *c) {
+    if (c->panel_mfma) {
+        if (c->dtype == SDDMM_BF16) launch_panel_mfma_steps<true>(c);
+        else launch_panel_mfma_steps<false>(c);
+        return;
+    }
     const Shape s = shape_of(c);
     if (s.unit == 0) launch_panel_u<UnitF32x4>(c, s);
     else launch_panel_t<UnitBF16x8, 1>(c, s.KU);

@@ -51,7 +51,7 @@ def test_full_size(engine_factory, name, K, other):
     e.run()
     fixed = e.values()
     assert O.check_values(fixed, ref, mag=mag)[0]
-    if st.mfma_tiles == 0:
+    if st.mfma_tiles == 0 and st.panels == 0:        # only gather kernels: same per-entry arithmetic
         np.testing.assert_array_equal(fixed.view(np.uint32), auto.view(np.uint32))
     # the exact-order kernel is the CPU loop bit for bit, also at this size
     e.plan(capi.EXACT)

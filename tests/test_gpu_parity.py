@@ -420,7 +420,7 @@ def test_tile_path_not_applicable_falls_back_to_gather(engine_factory):
     assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B)
 
 
-def test_fem_blocks_tiles_and_panels(engine_factory):
+def test_fem_blocks_tiles_and_panels(engine_factory, monkeypatch):
     w = W.make("fem_banded", "small")
     got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.MFMA_TILE)
     assert st.nnz_mfma == w.nnz and st.mfma_tiles == _tile_count(w.rowptr, w.col, w.M)
@@ -428,9 +428,14 @@ def test_fem_blocks_tiles_and_panels(engine_factory):
     # every block row is an 8-row panel with one column list
     got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.LDS_TILED)
     assert st.panels == w.M // 8 and st.nnz_panel == w.nnz and st.mfma_tiles == 0
-    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem panels")
+    assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem panels (MFMA kernel)")
+    # the VALU panel kernel has the per-entry arithmetic of the gather kernels
+    monkeypatch.setenv("SDDMM_PANEL_MFMA", "0")
+    got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.LDS_TILED)
+    assert st.panels == w.M // 8 and st.nnz_panel == w.nnz
     flat, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.FLAT)
-    np.testing.assert_array_equal(got.view(np.uint32), flat.view(np.uint32))   # same per-entry arithmetic
+    np.testing.assert_array_equal(got.view(np.uint32), flat.view(np.uint32))
+    monkeypatch.delenv("SDDMM_PANEL_MFMA")
     got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
     assert st.nnz_mfma + st.nnz_panel == w.nnz
     assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, what="fem auto")
@@ -438,7 +443,7 @@ def test_fem_blocks_tiles_and_panels(engine_factory):
 
 @pytest.mark.parametrize("K,dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (64, "bf16"), (256, "bf16"),
                                      (24, "f32"), (33, "f32")])
-def test_row_panels(engine_factory, K, dtype):
+def test_row_panels(engine_factory, monkeypatch, K, dtype):
     """Groups of identical rows: aligned 8-row panels are taken, everything else
     (unaligned groups, groups of other sizes, rows with one differing column, short
     lists, the ragged tail) stays on the row kernels."""
@@ -476,7 +481,9 @@ def test_row_panels(engine_factory, K, dtype):
         ops, dt = (Ab, Bb), capi.BF16
     else:
         ops, dt = (A, B), capi.F32
-    applicable = (dtype, K) in (("f32", 32), ("f32", 64), ("bf16", 64))     # A rows of a panel fit in registers
+    row_bytes = K * (2 if dtype == "bf16" else 4)
+    applicable = row_bytes % 64 == 0                                         # the MFMA panel kernel
+    valu_applicable = (dtype, K) in (("f32", 32), ("f32", 64), ("bf16", 64))  # A rows of a panel fit in registers
     same = len(rows_cols[51]) == 50 and np.array_equal(rows_cols[51], rows_cols[48])
     assert not same
     for strategy, min_len in ((capi.LDS_TILED, 1), (capi.AUTO, 16)):
@@ -487,7 +494,9 @@ def test_row_panels(engine_factory, K, dtype):
             exp = [(0, 300), (8, 70), (32, 33), (40, 33), (56, 9)] if applicable else []
             assert st.panels == len(exp) and st.nnz_panel == sum(8 * l for _, l in exp)
             assert st.mfma_tiles == 0
-    if applicable:
-        flat, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.FLAT, dt)
-        lds, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.LDS_TILED, dt)
-        np.testing.assert_array_equal(flat.view(np.uint32), lds.view(np.uint32))
+    monkeypatch.setenv("SDDMM_PANEL_MFMA", "0")
+    lds, st = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.LDS_TILED, dt)
+    assert_parity(lds, rowptr, col, val, A, B, what="VALU panels K=%d" % K)
+    assert (st.panels == 5) == valu_applicable and (st.panels == 0) == (not valu_applicable)
+    flat, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.FLAT, dt)
+    np.testing.assert_array_equal(flat.view(np.uint32), lds.view(np.uint32))
