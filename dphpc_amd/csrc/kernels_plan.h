@@ -6,11 +6,11 @@
 
 namespace sddmm {
 
+// Host-side summary of what the structure kernels counted.
 struct PlanCounters {
     unsigned int bad_pattern;      // != 0: malformed CSR/COO
     unsigned int coo_unsorted;     // != 0: COO rows not non-decreasing
     unsigned int max_len;          // longest row
-    unsigned int pad;
     unsigned long long rows_nonempty;
     unsigned long long rows_short, rows_medium, rows_long;
     unsigned long long nnz_short, nnz_medium, nnz_long;
@@ -18,6 +18,46 @@ struct PlanCounters {
     unsigned long long n_tiles, nnz_tiles, tiles_scanned;     // dense-tile path
     unsigned long long n_panels, nnz_panels, panel_items;     // row-panel path
 };
+
+// The same counters on the device.  Sums that thousands of workgroups contribute to
+// are spread over SPREAD slots chosen by workgroup id (same-address atomics were
+// measured at ~10 ns each, which made the counting kernels atomic-bound); the host
+// adds the slots up after the copy.
+constexpr int SPREAD = 64;
+enum CounterKind {
+    K_ROWS_NONEMPTY = 0,
+    K_ROWS_SHORT, K_ROWS_MEDIUM, K_ROWS_LONG, K_NNZ_SHORT, K_NNZ_MEDIUM, K_NNZ_LONG,   // row classifier
+    K_TILES, K_NNZ_TILES, K_PANELS, K_NNZ_PANELS,                                      // ownership classifiers
+    K_KINDS
+};
+struct DevCounters {
+    unsigned int bad_pattern, coo_unsorted, pad0, pad1;
+    unsigned long long n_items, tiles_scanned, panel_items, pad2;   // scan totals, one writer each
+    unsigned int max_len[SPREAD];
+    unsigned long long k[K_KINDS][SPREAD];
+};
+
+__device__ __forceinline__ void spread_add(DevCounters *dc, int kind, unsigned long long v) {
+    if (v) atomicAdd(&dc->k[kind][blockIdx.x & (SPREAD - 1)], v);
+}
+
+inline PlanCounters summarize(const DevCounters &d) {
+    PlanCounters p{};
+    p.bad_pattern = d.bad_pattern;
+    p.coo_unsorted = d.coo_unsorted;
+    unsigned long long sum[K_KINDS] = {0};
+    for (int s = 0; s < SPREAD; ++s) {
+        p.max_len = d.max_len[s] > p.max_len ? d.max_len[s] : p.max_len;
+        for (int k = 0; k < K_KINDS; ++k) sum[k] += d.k[k][s];
+    }
+    p.rows_nonempty = sum[K_ROWS_NONEMPTY];
+    p.rows_short = sum[K_ROWS_SHORT]; p.rows_medium = sum[K_ROWS_MEDIUM]; p.rows_long = sum[K_ROWS_LONG];
+    p.nnz_short = sum[K_NNZ_SHORT]; p.nnz_medium = sum[K_NNZ_MEDIUM]; p.nnz_long = sum[K_NNZ_LONG];
+    p.n_tiles = sum[K_TILES]; p.nnz_tiles = sum[K_NNZ_TILES];
+    p.n_panels = sum[K_PANELS]; p.nnz_panels = sum[K_NNZ_PANELS];
+    p.n_items = d.n_items; p.tiles_scanned = d.tiles_scanned; p.panel_items = d.panel_items;
+    return p;
+}
 
 __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
@@ -32,9 +72,12 @@ __device__ __forceinline__ unsigned int wave_max_u32(unsigned int v) {
 }
 
 // rowptr[0]==0, rowptr[M]==nnz, non-decreasing; also counts non-empty rows and the
-// longest row.  One lane per row.
+// longest row.  One lane per row, one set of atomics per workgroup.
 __global__ __launch_bounds__(256) void k_check_rowptr(const int32_t *__restrict__ rowptr, int M,
-                                                      int64_t nnz, PlanCounters *pc) {
+                                                      int64_t nnz, DevCounters *pc) {
+    __shared__ unsigned int sh_ne, sh_mx, sh_bad;
+    if (threadIdx.x == 0) { sh_ne = 0; sh_mx = 0; sh_bad = 0; }
+    __syncthreads();
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     unsigned int bad = 0, len = 0;
     if (i < M) {
@@ -43,19 +86,25 @@ __global__ __launch_bounds__(256) void k_check_rowptr(const int32_t *__restrict_
         if (i == 0 && s != 0) bad = 1;
         if (i == M - 1 && (int64_t)e != nnz) bad = 1;
     }
-    const unsigned long long ne = wave_sum_u64(len > 0 ? 1ull : 0ull);
+    const unsigned int ne = (unsigned int)__builtin_popcountll(__ballot(len > 0));
     const unsigned int mx = wave_max_u32(len);
     const unsigned long long anybad = __ballot(bad != 0);
     if (lane_id() == 0) {
-        if (ne) atomicAdd(&pc->rows_nonempty, ne);
-        if (mx) atomicMax(&pc->max_len, mx);
-        if (anybad) atomicOr(&pc->bad_pattern, 1u);
+        if (ne) atomicAdd(&sh_ne, ne);
+        if (mx) atomicMax(&sh_mx, mx);
+        if (anybad) atomicOr(&sh_bad, 1u);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        spread_add(pc, K_ROWS_NONEMPTY, sh_ne);
+        if (sh_mx) atomicMax(&pc->max_len[blockIdx.x & (SPREAD - 1)], sh_mx);
+        if (sh_bad) atomicOr(&pc->bad_pattern, 1u);
     }
 }
 
 // every column index in [0,N)
 __global__ __launch_bounds__(256) void k_check_index(const int32_t *__restrict__ idx, int64_t n,
-                                                     int bound, PlanCounters *pc) {
+                                                     int bound, DevCounters *pc) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     unsigned int bad = 0;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
@@ -91,7 +140,7 @@ __global__ __launch_bounds__(256) void k_expand_rows(const int32_t *__restrict__
 
 // COO rows non-decreasing?  (one lane per entry)
 __global__ __launch_bounds__(256) void k_check_coo_sorted(const int32_t *__restrict__ row, int64_t nnz,
-                                                          PlanCounters *pc) {
+                                                          DevCounters *pc) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     unsigned int uns = 0;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i + 1 < nnz; i += stride)
@@ -165,7 +214,7 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
                                                                const unsigned char *__restrict__ owner8, int M,
                                                                int ts, int seg, unsigned int *__restrict__ block_sums,
-                                                               PlanCounters *pc) {
+                                                               DevCounters *pc) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int items = 0;
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
@@ -181,16 +230,22 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__
     unsigned int total;
     (void)block_exclusive_scan(items, &total);
     if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+    // statistics: wave sums, then one set of atomics per workgroup
+    __shared__ unsigned long long sh[6];
+    if (threadIdx.x < 6) sh[threadIdx.x] = 0;
+    __syncthreads();
     r_short = wave_sum_u64(r_short); r_med = wave_sum_u64(r_med); r_long = wave_sum_u64(r_long);
     n_short = wave_sum_u64(n_short); n_med = wave_sum_u64(n_med); n_long = wave_sum_u64(n_long);
     if (lane_id() == 0) {
-        if (r_short) atomicAdd(&pc->rows_short, r_short);
-        if (r_med) atomicAdd(&pc->rows_medium, r_med);
-        if (r_long) atomicAdd(&pc->rows_long, r_long);
-        if (n_short) atomicAdd(&pc->nnz_short, n_short);
-        if (n_med) atomicAdd(&pc->nnz_medium, n_med);
-        if (n_long) atomicAdd(&pc->nnz_long, n_long);
+        if (r_short) atomicAdd(&sh[0], r_short);
+        if (r_med) atomicAdd(&sh[1], r_med);
+        if (r_long) atomicAdd(&sh[2], r_long);
+        if (n_short) atomicAdd(&sh[3], n_short);
+        if (n_med) atomicAdd(&sh[4], n_med);
+        if (n_long) atomicAdd(&sh[5], n_long);
     }
+    __syncthreads();
+    if (threadIdx.x < 6) spread_add(pc, K_ROWS_SHORT + (int)threadIdx.x, sh[threadIdx.x]);
 }
 
 // pass 2: exclusive scan of the block sums in place (one workgroup), total -> *total_out
@@ -243,7 +298,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
 __global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__ rowptr,
                                                      const int32_t *__restrict__ col, int M, int64_t n_panels,
                                                      int min_len, int pseg, unsigned char *__restrict__ owner8,
-                                                     unsigned int *__restrict__ counts, PlanCounters *pc) {
+                                                     unsigned int *__restrict__ counts, DevCounters *pc) {
     const int64_t p = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     if (p >= n_panels) return;
     const int lane = lane_id();
@@ -256,12 +311,18 @@ __global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__
         ok = len >= min_len;
         for (int r = 1; ok && r < 8; ++r) ok = rowptr[row0 + r + 1] - rowptr[row0 + r] == len;
     }
-    // ok is the same in every lane here
+    // ok is the same in every lane here.  Equal lengths make the 8 rows equally spaced
+    // in the CSR arrays (row r starts at s0 + r*len), so the 7 comparisons of one
+    // position are independent loads.
     if (ok) {
         bool differ = false;
         for (int e = lane; e < len; e += WAVE) {
-            const int c0 = col[s0 + e];
-            for (int r = 1; r < 8; ++r) differ |= col[rowptr[row0 + r] + e] != c0;
+            const int32_t *pc0 = col + s0 + e;
+            const int c0 = pc0[0];
+            int d = 0;
+#pragma unroll
+            for (int r = 1; r < 8; ++r) d |= pc0[(int64_t)r * len] ^ c0;
+            differ |= d != 0;
         }
         ok = __ballot(differ) == 0;
     }
@@ -269,8 +330,8 @@ __global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__
         counts[p] = ok ? (unsigned int)((len + pseg - 1) / pseg) : 0u;
         if (ok) {
             owner8[p] = 2;
-            atomicAdd(&pc->n_panels, 1ull);
-            atomicAdd(&pc->nnz_panels, (unsigned long long)len * 8ull);
+            spread_add(pc, K_PANELS, 1ull);
+            spread_add(pc, K_NNZ_PANELS, (unsigned long long)len * 8ull);
         }
     }
 }

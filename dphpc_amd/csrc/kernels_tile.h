@@ -60,6 +60,8 @@ __device__ __forceinline__ int sum16(int v) {
 // row's first position and column mask in the tile (mask 0: row absent).  The walk
 // stops early when on_tile returns false (it must return the same in all 16 lanes).
 // Returns false in a lane whose row is not strictly increasing in column.
+struct __attribute__((packed, aligned(4))) I4u { int x, y, z, w; };
+
 template <class F>
 __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M,
                                            int64_t strip, int sub, F &&on_tile) {
@@ -68,7 +70,34 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
     if (row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
     bool sorted = true;
     int prev = -1;
-    int c = p < end ? col[p] : -1;
+    // The row is read 8 column indices at a time (two 16-byte loads, clamped to the
+    // row's last entry), so the walk is not one dependent load per entry.
+    int buf[8];
+    int buf_at = p;                       // buf[i] = col[min(buf_at + i, end - 1)]
+    auto refill = [&](int at) {
+        buf_at = at;
+        if (at < end) {
+            const int last = end - 1;
+            if (at + 7 <= last) {
+                const I4u lo = *reinterpret_cast<const I4u *>(col + at);
+                const I4u hi = *reinterpret_cast<const I4u *>(col + at + 4);
+                buf[0] = lo.x; buf[1] = lo.y; buf[2] = lo.z; buf[3] = lo.w;
+                buf[4] = hi.x; buf[5] = hi.y; buf[6] = hi.z; buf[7] = hi.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) buf[i] = col[at + i < last ? at + i : last];
+            }
+        }
+    };
+    auto peek = [&](int at) {             // col[at] for buf_at <= at < buf_at + 8
+        const int i = at - buf_at;
+        int v = buf[0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) v = i == k ? buf[k] : v;
+        return v;
+    };
+    refill(p);
+    int c = p < end ? peek(p) : -1;
     while (true) {
         const int mine = p < end ? (c >> 4) : INT32_MAX;
         const int t = min16(mine);
@@ -80,7 +109,8 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
             prev = c;
             mask |= 1u << (c & 15);
             ++p;
-            c = p < end ? col[p] : -1;
+            if (p - buf_at >= 8) refill(p);
+            c = p < end ? peek(p) : -1;
         }
         if (!on_tile(t, first, mask)) break;
     }
@@ -93,7 +123,7 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
 __global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ rowptr,
                                                     const int32_t *__restrict__ col, int M, int64_t n_strips,
                                                     int min_fill, unsigned int *__restrict__ strip_ntiles,
-                                                    unsigned char *__restrict__ owner8, PlanCounters *pc) {
+                                                    unsigned char *__restrict__ owner8, DevCounters *pc) {
     const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int sub = threadIdx.x & 15;
     if (strip >= n_strips) return;   // whole 16-lane rows leave together
@@ -117,8 +147,8 @@ __global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ 
         if (take) {
             owner8[2 * strip] = 1;         // both 8-row halves (the array is padded to an even length)
             owner8[2 * strip + 1] = 1;
-            atomicAdd(&pc->n_tiles, (unsigned long long)tiles);
-            atomicAdd(&pc->nnz_tiles, (unsigned long long)all_entries);
+            spread_add(pc, K_TILES, (unsigned long long)tiles);
+            spread_add(pc, K_NNZ_TILES, (unsigned long long)all_entries);
         }
     }
 }

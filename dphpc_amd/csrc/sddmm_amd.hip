@@ -44,8 +44,9 @@ struct sddmm_ctx {
     bool planned = false;
     int strategy = SDDMM_AUTO;       // resolved
     int requested = SDDMM_AUTO;
-    PlanCounters *d_pc = nullptr;    // device counters
-    PlanCounters pc{};               // host copy
+    DevCounters *d_pc = nullptr;     // device counters
+    DevCounters raw{};               // host copy of the device block
+    PlanCounters pc{};               // its summary
     sddmm_stats stats{};
     // AUTO: rows shorter than ts go to the many-rows-per-wave kernel, the others
     // become wave-per-segment items of at most seg entries
@@ -155,8 +156,9 @@ int grid_capped(int64_t n, int block, int cap = 16384) {
 }
 
 int fetch_counters(sddmm_ctx *c) {
-    HIP_TRY(c, hipMemcpyAsync(&c->pc, c->d_pc, sizeof(PlanCounters), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, hipMemcpyAsync(&c->raw, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(c, hipStreamSynchronize(c->stream));
+    c->pc = summarize(c->raw);
     return SDDMM_OK;
 }
 
@@ -309,13 +311,10 @@ int classify_rows(sddmm_ctx *c) {
         ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
         c->block_sums_cap = nb;
     }
-    // keep what validation measured, clear what the classifier accumulates
-    PlanCounters fresh = c->pc;
-    fresh.rows_short = fresh.rows_medium = fresh.rows_long = 0;
-    fresh.nnz_short = fresh.nnz_medium = fresh.nnz_long = 0;
-    fresh.n_items = 0;
-    c->pc = fresh;
-    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
+    // keep what validation and the ownership classifiers measured, clear the row classes
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
+                              sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     if (nb > 0) {
         const unsigned char *owner = c->owner_active ? c->d_owner8 : nullptr;
         hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, owner,
@@ -369,9 +368,9 @@ int begin_ownership(sddmm_ctx *c) {
         c->owner_cap = bytes;
     }
     HIP_TRY(c, hipMemsetAsync(c->d_owner8, 0, (size_t)bytes, c->stream));
-    c->pc.n_tiles = c->pc.nnz_tiles = c->pc.tiles_scanned = 0;
-    c->pc.n_panels = c->pc.nnz_panels = c->pc.panel_items = 0;
-    HIP_TRY(c, hipMemcpyAsync(c->d_pc, &c->pc, sizeof(PlanCounters), hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_TILES][0], 0,
+                              sizeof(unsigned long long) * SPREAD * (K_NNZ_PANELS - K_TILES + 1), c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 2 * sizeof(unsigned long long), c->stream));
     c->owner_active = true;
     c->tiles_active = false;
     c->n_tiles = c->nnz_tiles = 0;
@@ -555,7 +554,7 @@ int ensure_rowidx(sddmm_ctx *c) {
 
 // Validate the device-resident CSR and gather row statistics.
 int validate_csr(sddmm_ctx *c) {
-    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
     if (c->sM > 0)
         hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(c->sM, 256)), dim3(256), 0, c->stream, c->d_rowptr, c->sM,
                            c->nnz, c->d_pc);
@@ -731,7 +730,7 @@ int sddmm_create(sddmm_ctx **out, int device) {
     if (!c) return SDDMM_ERR_ALLOC;
     c->device = device;
     if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
-        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(PlanCounters)) != hipSuccess) {
+        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(DevCounters)) != hipSuccess) {
         sddmm_destroy(c);
         return SDDMM_ERR_HIP;
     }
@@ -852,7 +851,7 @@ int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, c
     ALLOC_TRY(c, c->dP, (size_t)nnz * sizeof(float));
     ALLOC_TRY(c, c->d_rowptr, (size_t)(M + 1) * sizeof(int32_t));
     c->sM = M; c->sN = N; c->nnz = nnz;
-    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+    HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
     if (nnz) {
         HIP_TRY(c, hipMemcpyAsync(c->d_rowidx, row, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
         HIP_TRY(c, hipMemcpyAsync(c->d_col, col, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
@@ -875,7 +874,7 @@ int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, c
         hipLaunchKernelGGL(k_rowptr_from_sorted_coo, dim3(grid_for(nnz + 1, 256)), dim3(256), 0, c->stream,
                            c->d_rowidx, nnz, M, c->d_rowptr);
         HIP_TRY(c, hipGetLastError());
-        HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(PlanCounters), c->stream));
+        HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
         if (M > 0)
             hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(M, 256)), dim3(256), 0, c->stream, c->d_rowptr, M, nnz,
                                c->d_pc);
