@@ -133,7 +133,8 @@ int main(int argc, char **argv) {
     }
     if (K < 1 || num_runs < 1 || scale <= 0) { std::fprintf(stderr, "bad arguments\n"); return 2; }
     std::vector<std::shared_ptr<Competitors::GPUAmd>> comps;
-    for (int st : {SDDMM_EXACT, SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE}) comps.push_back(std::make_shared<Competitors::GPUAmd>(st));
+    for (int st : {SDDMM_EXACT, SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_SHORT_ROWS, SDDMM_LDS_TILED, SDDMM_MFMA_TILE})
+        comps.push_back(std::make_shared<Competitors::GPUAmd>(st));
     if (header)
         std::cout << "competitor,dataset,mat_repr,M,N,K,NZ,total_ns,init_ns,comp_ns,cleanup_ns,correctness,num_thread_blocks,num_threads_per_block" << std::endl;
     auto want = [&](const char *n) { return only.empty() || only == n; };

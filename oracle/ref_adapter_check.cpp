@@ -83,7 +83,7 @@ static void compare(std::vector<std::shared_ptr<SDDMM::Competitor<float>>> &comp
 int main() {
     std::vector<std::shared_ptr<SDDMM::Competitor<float>>> comps;
     comps.push_back(std::make_shared<Competitors::CPUBasic<float>>());
-    for (int st : {SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_EXACT})
+    for (int st : {SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_SHORT_ROWS, SDDMM_LDS_TILED, SDDMM_MFMA_TILE, SDDMM_EXACT})
         comps.push_back(std::make_shared<Competitors::GPUAmd>(st));
     std::mt19937_64 rng(2024);
     {

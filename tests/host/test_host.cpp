@@ -166,7 +166,7 @@ static void cpu_cases() {
 }
 
 // ---------------------------------------------------------------- GPU cases
-static const int kStrategies[] = {SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_EXACT};
+static const int kStrategies[] = {SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_SHORT_ROWS, SDDMM_LDS_TILED, SDDMM_MFMA_TILE, SDDMM_EXACT};
 
 // tests/matrix_test.cc:40-59 with the oracle in the role of float_competitors[0]
 // `harness_predicate`: also apply the containers' operator== (1e-3 relative to the

@@ -63,7 +63,8 @@ def test_driver_prints_reference_csv_and_all_runs_are_correct():
     assert p.returncode == 0, p.stdout
     rows = _csv_rows(p.stdout)
     assert {r["dataset"] for r in rows} == {"small_uniform", "fem_banded", "power_law", "mixed_density", "dense_tiles"}
-    assert {r["competitor"] for r in rows} == {"GPU-AMD-Exact", "GPU-AMD-Dynamic", "GPU-AMD-Flat", "GPU-AMD-RowWave"}
+    assert {r["competitor"] for r in rows} == {"GPU-AMD-Exact", "GPU-AMD-Dynamic", "GPU-AMD-Flat", "GPU-AMD-RowWave",
+                                               "GPU-AMD-ShortRows", "GPU-AMD-Tiled", "GPU-AMD-MFMA"}
     assert {r["mat_repr"] for r in rows} == {"CSR", "COO"}
     for r in rows:
         assert r["correctness"] == "1", r
