@@ -364,7 +364,9 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
     const int lane = lane_id();
     const int n = lane & 15, q = lane >> 4;
     constexpr int ROW_UNITS = STEPS * 4;
-    constexpr int GROUPS = 4;                                   // groups of 16 columns per chunk
+    // groups of 16 columns in flight; 1, 2 and 4 measured the same (47-50 us on the
+    // FEM shape at K=32): the kernel is not bound by its own prefetch depth
+    constexpr int GROUPS = 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored
@@ -433,19 +435,20 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
         }
     };
 
+    constexpr int CHUNK = GROUPS * 16;                          // columns per loop iteration (<= 64)
     Oper o[GROUPS];
     {
         const int cc0 = cols_of_chunk(start);
 #pragma unroll
         for (int u = 0; u < GROUPS; ++u) o[u] = load_oper(__shfl(cc0, u * 16 + n, WAVE), start + 16 * u);
     }
-    int cc_nxt = cols_of_chunk(start + WAVE);                   // columns of the next chunk
-    for (int base = start; base < end; base += WAVE) {
-        const int cc_nn = cols_of_chunk(base + 2 * WAVE);
+    int cc_nxt = cols_of_chunk(start + CHUNK);                  // columns of the next chunk
+    for (int base = start; base < end; base += CHUNK) {
+        const int cc_nn = cols_of_chunk(base + 2 * CHUNK);
 #pragma unroll
         for (int u = 0; u < GROUPS; ++u) {
             compute_store(o[u], base + 16 * u);
-            o[u] = load_oper(__shfl(cc_nxt, u * 16 + n, WAVE), base + WAVE + 16 * u);
+            o[u] = load_oper(__shfl(cc_nxt, u * 16 + n, WAVE), base + CHUNK + 16 * u);
         }
         cc_nxt = cc_nn;
     }
