@@ -418,7 +418,7 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
                        c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
     HIP_TRY(c, hipGetLastError());
     c->tiles_active = true;
-    c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 8));
+    c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 4));
     return SDDMM_OK;
 }
 
