@@ -192,4 +192,36 @@ inline bool read_matrix_market(const std::string &path, int K, uint64_t seed, Da
     return true;
 }
 
+// SNAP edge list reader (the format of EMailEnronDataset,
+// src/benchmark/dataset.hpp:271-313): leading '#' comment lines (the reference
+// skips the first four lines, which is what SNAP files carry), then one
+// "row<TAB>col" pair per line with 0-based indices; every edge gets value 1 and
+// the edge list is taken as directed, exactly as written.  dim > 0 fixes the
+// square dimension (36692 for email-Enron in the reference); dim == 0 takes
+// 1 + the largest index seen.  Returns false when the file cannot be parsed.
+inline bool read_snap_edge_list(const std::string &path, int dim, int K, uint64_t seed, Dataset &out, std::string &err) {
+    std::ifstream in(path);
+    if (!in) { err = "cannot open " + path; return false; }
+    std::vector<Triplet<float>> t;
+    std::string line;
+    long long top = -1, lineno = 0;
+    while (std::getline(in, line)) {
+        ++lineno;
+        if (line.empty() || line[0] == '#' || line[0] == '%') continue;
+        std::istringstream e(line);
+        long long r, c;
+        if (!(e >> r >> c)) { err = "bad edge at line " + std::to_string(lineno); return false; }
+        if (r < 0 || c < 0 || r > 2147483646LL || c > 2147483646LL) { err = "index out of range at line " + std::to_string(lineno); return false; }
+        if (dim > 0 && (r >= dim || c >= dim)) { err = "index beyond the given dimension at line " + std::to_string(lineno); return false; }
+        top = std::max(top, std::max(r, c));
+        t.push_back({(int)r, (int)c, 1.f});
+    }
+    if (t.empty()) { err = "no edges"; return false; }
+    const int n = dim > 0 ? dim : (int)(top + 1);
+    std::mt19937_64 rng(seed);
+    const size_t slash = path.find_last_of('/');
+    out = finish(slash == std::string::npos ? path : path.substr(slash + 1), n, n, K, std::move(t), rng, false);
+    return true;
+}
+
 }  // namespace sddmm_host

@@ -1,7 +1,7 @@
 // Benchmark driver for the GPUAmd competitor: the role of the reference's
 // src/main.cpp + src/benchmark/benchmark.hpp for this one competitor family.
 //
-//   sddmm_driver [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx] [--no_csv_header]
+//   sddmm_driver [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx|edges.txt] [--dim n] [--no_csv_header]
 //
 // Prints one CSV line per run in the reference's 14-column schema
 // (src/main.cpp:356-358, src/benchmark/benchmark.hpp:95-98):
@@ -120,6 +120,7 @@ int main(int argc, char **argv) {
     int K = 32, num_runs = 3;
     double scale = 0.1;
     bool header = true;
+    int snap_dim = 0;
     std::string only;
     for (int i = 1; i < argc; ++i) {
         const std::string a = argv[i];
@@ -128,8 +129,9 @@ int main(int argc, char **argv) {
         else if (a == "--num_runs") num_runs = std::atoi(next());
         else if (a == "--scale") scale = std::atof(next());
         else if (a == "--dataset" || a == "-d") only = next();
+        else if (a == "--dim") snap_dim = std::atoi(next());
         else if (a == "--no_csv_header") header = false;
-        else { std::fprintf(stderr, "usage: %s [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx] [--no_csv_header]\n", argv[0]); return 2; }
+        else { std::fprintf(stderr, "usage: %s [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx|edges.txt] [--dim n] [--no_csv_header]\n", argv[0]); return 2; }
     }
     if (K < 1 || num_runs < 1 || scale <= 0) { std::fprintf(stderr, "bad arguments\n"); return 2; }
     std::vector<std::shared_ptr<Competitors::GPUAmd>> comps;
@@ -144,6 +146,14 @@ int main(int argc, char **argv) {
         Dataset d;
         std::string err;
         if (!sddmm_host::read_matrix_market(only, K, seed, d, err)) { std::fprintf(stderr, "%s: %s\n", only.c_str(), err.c_str()); return 1; }
+        bench_dataset(d, comps, num_runs);
+        return 0;
+    }
+    if (only.size() > 4 && only.substr(only.size() - 4) == ".txt") {
+        // SNAP edge list, e.g. email-Enron.txt --dim 36692 (src/benchmark/dataset.hpp:271-313)
+        Dataset d;
+        std::string err;
+        if (!sddmm_host::read_snap_edge_list(only, snap_dim, K, seed, d, err)) { std::fprintf(stderr, "%s: %s\n", only.c_str(), err.c_str()); return 1; }
         bench_dataset(d, comps, num_runs);
         return 0;
     }

@@ -7,6 +7,8 @@
 //   test_host cpu   containers, conversions, partition vectors (no GPU needed)
 //   test_host gpu   everything that launches kernels
 #include <cstdio>
+#include <cstdlib>
+#include <unistd.h>
 #include <cstring>
 #include <memory>
 #include <random>
@@ -14,6 +16,7 @@
 #include <vector>
 
 #include "gpu_amd.hpp"
+#include "datasets.hpp"
 
 extern "C" {
 void oracle_sddmm_csr_f32(int M, int K, const int32_t *rowptr, const int32_t *col, const float *sval,
@@ -162,6 +165,46 @@ static void cpu_cases() {
         CSR<float> zero(x), zero2(x);
         zero.clearValues(); zero2.clearValues();
         CHECK(zero == zero2);               // 0/0 is NaN in the reference
+    }
+    {
+        CASE("file_readers");   // src/benchmark/dataset.hpp:123-181 (Matrix Market), :271-313 (SNAP edge list)
+        char dir[] = "/tmp/sddmm_host_XXXXXX";
+        CHECK(mkdtemp(dir) != nullptr);
+        const std::string base(dir);
+        auto put = [&](const char *name, const char *text) {
+            std::ofstream f(base + "/" + name);
+            f << text;
+            return base + "/" + name;
+        };
+        sddmm_host::Dataset d;
+        std::string err;
+        // four header lines, TAB-separated 0-based pairs, a repeated edge, directed as written
+        const std::string snap = put("edges.txt", "# Directed graph\n# tiny\n# Nodes: 5 Edges: 5\n# FromNodeId\tToNodeId\n"
+                                                  "0\t1\n3\t0\n1\t4\n0\t1\n4\t4\n");
+        CHECK(sddmm_host::read_snap_edge_list(snap, 0, 8, 7, d, err));
+        CHECK(d.S_csr.getRows() == 5 && d.S_csr.getCols() == 5 && d.A.getRows() == 5 && d.B.getCols() == 8);
+        CHECK((d.S_csr.getRowPositions() == std::vector<int>{0, 1, 2, 2, 3, 4}));   // the repeated edge is stored once
+        CHECK((d.S_csr.getColPositions() == std::vector<int>{1, 4, 0, 4}));
+        CHECK((d.S_csr.getValues() == std::vector<float>{1.f, 1.f, 1.f, 1.f}));
+        CHECK(d.S_coo.getRowPositions() == (std::vector<int>{0, 1, 3, 4}));
+        CHECK(sddmm_host::read_snap_edge_list(snap, 36, 4, 7, d, err) && d.S_csr.getRows() == 36 && d.S_csr.getCols() == 36);
+        CHECK(!sddmm_host::read_snap_edge_list(snap, 4, 4, 7, d, err) && err.find("dimension") != std::string::npos);
+        CHECK(!sddmm_host::read_snap_edge_list(put("bad.txt", "# x\n1\n"), 0, 4, 7, d, err));
+        CHECK(!sddmm_host::read_snap_edge_list(base + "/absent.txt", 0, 4, 7, d, err));
+        // Matrix Market: 1-based, symmetric not expanded, pattern -> 1, tiny values dropped
+        const std::string mm = put("m.mtx", "%%MatrixMarket matrix coordinate real symmetric\n% c\n3 4 4\n"
+                                            "1 1 2.5\n3 4 -1\n2 2 1e-9\n2 1 0.5\n");
+        CHECK(sddmm_host::read_matrix_market(mm, 4, 7, d, err));
+        CHECK(d.S_csr.getRows() == 3 && d.S_csr.getCols() == 4);
+        CHECK((d.S_csr.getRowPositions() == std::vector<int>{0, 1, 2, 3}));
+        CHECK((d.S_csr.getColPositions() == std::vector<int>{0, 0, 3}));
+        CHECK((d.S_csr.getValues() == std::vector<float>{2.5f, 0.5f, -1.f}));
+        const std::string pat = put("p.mtx", "%%MatrixMarket matrix coordinate pattern general\n2 2 2\n2 1\n1 2\n");
+        CHECK(sddmm_host::read_matrix_market(pat, 4, 7, d, err));
+        CHECK((d.S_csr.getValues() == std::vector<float>{1.f, 1.f}) && (d.S_csr.getColPositions() == std::vector<int>{1, 0}));
+        CHECK(!sddmm_host::read_matrix_market(put("a.mtx", "%%MatrixMarket matrix array real general\n2 2\n1\n2\n3\n4\n"), 4, 7, d, err));
+        for (const char *n : {"edges.txt", "bad.txt", "m.mtx", "p.mtx", "a.mtx"}) std::remove((base + "/" + n).c_str());
+        rmdir(dir);
     }
 }
 

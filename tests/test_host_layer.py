@@ -87,3 +87,22 @@ def test_driver_reads_matrix_market_like_the_reference(tmp_path):
     bad.write_text("%%MatrixMarket matrix coordinate real general\n2 2 2\n1 1 1.0\n")
     p = _run([DRIVER, "--dataset", str(bad)], 60)
     assert p.returncode == 1 and "ends before" in p.stdout
+
+
+@pytest.mark.gpu
+def test_driver_reads_snap_edge_list_like_the_reference(tmp_path):
+    # four '#' header lines, TAB-separated 0-based pairs, value 1, fixed square
+    # dimension (src/benchmark/dataset.hpp:271-313)
+    import random
+    rnd = random.Random(5)
+    edges = {(rnd.randrange(300), rnd.randrange(300)) for _ in range(4000)}
+    txt = tmp_path / "edges.txt"
+    txt.write_text("# Directed graph\n# test\n# Nodes: 300 Edges: %d\n# FromNodeId\tToNodeId\n" % len(edges)
+                   + "".join("%d\t%d\n" % e for e in sorted(edges)))
+    p = _run([DRIVER, "--dataset", str(txt), "--dim", "320", "--num_runs", "1", "--K", "32"], 60)
+    assert p.returncode == 0, p.stdout
+    rows = _csv_rows(p.stdout)
+    assert rows and all(r["M"] == "320" and r["N"] == "320" and r["NZ"] == str(len(edges)) and r["correctness"] == "1"
+                        for r in rows)
+    p = _run([DRIVER, "--dataset", str(txt), "--dim", "100"], 60)
+    assert p.returncode == 1 and "dimension" in p.stdout
