@@ -4,10 +4,10 @@
 //
 //   * a strip is rows [16*ti, 16*ti+16); a tile is the strip's entries whose
 //     column lies in [16*tj, 16*tj+16);
-//   * the classifier (k_tile_count / k_tile_fill, plan phase, device only) walks
-//     the sorted column lists of the 16 rows of a strip in step and emits one
-//     TileDesc per non-empty tile: for every row the CSR position of its first
-//     entry inside the tile and a 16-bit mask of the columns present;
+//   * the classifier (k_strip_count / k_strip_tiles / k_tile_rows, plan phase,
+//     device only) finds the non-empty tiles of every strip and emits one TileDesc
+//     per tile: for every row the CSR position of its first entry inside the tile
+//     and a 16-bit mask of the columns present;
 //   * a strip goes to this path as a whole (then every one of its entries is
 //     computed here, sparse tiles included) or not at all, so the gather kernels
 //     and this one never share a row;
@@ -117,61 +117,271 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
     return sorted;
 }
 
-// pass 1: tiles and entries per strip; a strip qualifies when all its rows are
-// sorted and it holds at least min_fill entries per tile on average.
-// strip_ntiles[s] = number of tiles (0: strip stays on the gather kernels).
-__global__ __launch_bounds__(256) void k_tile_count(const int32_t *__restrict__ rowptr,
-                                                    const int32_t *__restrict__ col, int M, int64_t n_strips,
-                                                    int min_fill, unsigned int *__restrict__ strip_ntiles,
-                                                    unsigned char *__restrict__ owner8, DevCounters *pc) {
-    const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
-    const int sub = threadIdx.x & 15;
-    if (strip >= n_strips) return;   // whole 16-lane rows leave together
-    // entries of the strip, known from rowptr alone: the walk can stop as soon as the
-    // strip has more tiles than that many entries could fill to the threshold
-    const int64_t r_lo = strip * 16, r_hi = r_lo + 16 < M ? r_lo + 16 : M;
-    const int64_t strip_entries = (int64_t)rowptr[r_hi] - (int64_t)rowptr[r_lo];
-    const int64_t max_tiles = strip_entries / min_fill;
-    int tiles = 0, entries = 0;
-    const bool sorted = walk_strip(rowptr, col, M, strip, sub, [&](int, int, unsigned int mask) {
-        ++tiles;
-        entries += __builtin_popcount(mask);
-        return (int64_t)tiles <= max_tiles;
-    });
-    const int all_entries = sum16(entries);
-    const int unsorted = sum16(sorted ? 0 : 1);
-    const bool take = unsorted == 0 && tiles > 0 && (int64_t)tiles <= max_tiles &&
-                      (int64_t)all_entries >= (int64_t)min_fill * tiles;
-    if (sub == 0) {
+// ---- parallel strip classifier ---------------------------------------------------
+// One wavefront per strip, four strips per workgroup.  The strip's entries are
+// contiguous in the CSR arrays, so the wave streams them 64 per load, several
+// loads in flight, instead of merging 16 sorted lists entry by entry:
+//
+//   * walking the entries in storage order, the tile column changes at least once
+//     per (row, tile) pair minus the 15 row boundaries, and a strip has at least
+//     (pairs / 16) tiles: the number of changes bounds the tile count from below
+//     without any merging, and the scan stops as soon as that bound exceeds what
+//     the fill threshold allows (a strip of scattered entries is given up after
+//     its first few hundred);
+//   * the same scan marks the tile column after every change in a bitmap in LDS
+//     that covers the strip's column span -- every tile present is marked at least
+//     once; the number of set bits is the number of tiles, the rank of a bit the
+//     position of its tile in the strip's (column-ordered) descriptor range;
+//   * rows are strictly increasing iff the only places where a column does not
+//     exceed its predecessor are row boundaries: the scan counts all such places,
+//     the 16 row starts are checked apart;
+//   * a strip whose span does not fit the bitmap is scanned without it and, if it
+//     passes, merged by the walk above in its first 16 lanes.
+//
+// The bitmap is private to its wave: LDS operations of one wave execute in program
+// order, so clearing, marking and counting need no workgroup barrier, only that
+// the compiler keeps their order (wave_lds_order).
+constexpr int STRIP_BM_WORDS = 1024;          // 32768 tile columns: a span of 524288 columns
+constexpr int STRIP_UNROLL = 8;               // loads of 64 entries per batch, two batches in flight
+constexpr int STRIPS_PER_BLOCK = 4;
+
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Streams entries [e0, e1).  Returns the number of tile-column changes, or -1 as
+// soon as it exceeds `budget`; *descents receives the number of entries whose
+// column does not exceed the column stored before them.  SET_BITS: also sets bit
+// (col>>4) - lo in bm after every change.
+template <bool SET_BITS>
+__device__ __forceinline__ int64_t strip_scan(const int32_t *__restrict__ col, int e0, int e1, int64_t budget,
+                                              int lo, int span, unsigned int *bm, int64_t *descents) {
+    const int lane = lane_id();
+    constexpr int BATCH = WAVE * STRIP_UNROLL;
+    int64_t changes = 0, desc = 0;
+    int carry = -1;                           // column before the batch; -1: entry e0 counts as a change
+    auto load = [&](int base, int (&c)[STRIP_UNROLL]) {
+#pragma unroll
+        for (int u = 0; u < STRIP_UNROLL; ++u) {
+            const int e = base + u * WAVE + lane;
+            if (base + u * WAVE < e1 || u == 0) c[u] = col[e < e1 ? e : e1 - 1];   // wave-uniform skip
+            else c[u] = 0;
+        }
+    };
+    int cur[STRIP_UNROLL], nxt[STRIP_UNROLL];
+    load(e0, cur);
+    for (int base = e0; base < e1; base += BATCH) {
+        load(base + BATCH, nxt);
+#pragma unroll
+        for (int u = 0; u < STRIP_UNROLL; ++u) {
+            const int cbase = base + u * WAVE;
+            if (cbase >= e1) break;                           // wave-uniform
+            const bool valid = cbase + lane < e1;
+            // column of the entry before: lane - 1 (wave_shr:1), lane 0 takes the carry
+            const int prev = __builtin_amdgcn_update_dpp(carry, cur[u], 0x138, 0xF, 0xF, false);
+            carry = __builtin_amdgcn_readlane(cur[u], WAVE - 1);
+            const bool change = valid && (cur[u] >> 4) != (prev >> 4);
+            if constexpr (SET_BITS) {
+                const int t = (cur[u] >> 4) - lo;
+                if (change && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
+            }
+            changes += __popcll(__ballot(change));
+            desc += __popcll(__ballot(valid && cur[u] <= prev));
+        }
+        if (changes > budget) return -1;
+#pragma unroll
+        for (int u = 0; u < STRIP_UNROLL; ++u) cur[u] = nxt[u];
+    }
+    *descents = desc;
+    return changes;
+}
+
+// From the first and last entry of each of the 16 rows (lane i < 16: row i, whose
+// rowptr is lane_rp): the strip's column span in tile columns, [lo, lo + span)
+// (exact when the rows are sorted; span <= 0 when they are not or no row has an
+// entry), and the number of row starts whose column does not exceed the column
+// stored before them -- the descents a sorted strip is allowed.
+__device__ __forceinline__ void strip_bounds(const int32_t *__restrict__ col, int lane_rp, int e0, int *lo, int *span,
+                                             int *boundary_descents) {
+    const int lane = lane_id();
+    const int nxt = __shfl_down(lane_rp, 1, WAVE);
+    const bool has = lane < 16 && nxt > lane_rp;
+    const int first_col = has ? col[lane_rp] : INT32_MAX;
+    const int last_col = has ? col[nxt - 1] : -1;
+    const int before = has && lane_rp > e0 ? col[lane_rp - 1] : -1;
+    const int l = __builtin_amdgcn_readfirstlane(min16(has ? first_col >> 4 : INT32_MAX));
+    const int hneg = __builtin_amdgcn_readfirstlane(min16(has ? -(last_col >> 4) : 1));
+    *lo = l;
+    *span = l == INT32_MAX ? 0 : -hneg - l + 1;
+    *boundary_descents = __popcll(__ballot(has && first_col <= before));
+}
+
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+// pass 1: strip_ntiles[s] = number of tiles of a strip that goes to the tile path
+// (sorted rows, at least min_fill entries per tile on average), else 0.
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips, int min_fill,
+    unsigned int *__restrict__ strip_ntiles, unsigned char *__restrict__ owner8, DevCounters *pc) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
+    const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
+    if (strip >= n_strips) return;            // whole waves leave
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const int64_t r = strip * 16 + lane;
+    const int lane_rp = rowptr[r < M ? r : M];
+    const int e0 = __builtin_amdgcn_readlane(lane_rp, 0), e1 = __builtin_amdgcn_readlane(lane_rp, 16);
+    const int64_t entries = (int64_t)e1 - (int64_t)e0;
+    const int64_t max_tiles = entries / min_fill;
+    // changes >= (row, tile) pairs - 15 and tiles >= pairs / 16
+    const int64_t budget = 16 * max_tiles;
+    int64_t tiles = 0, descents = 0;
+    bool take = false;
+    // most strips of a scattered matrix are given up on their first 512 entries,
+    // before anything else is read
+    constexpr int FIRST = WAVE * STRIP_UNROLL;
+    if (max_tiles > 0 &&
+        strip_scan<false>(col, e0, e1 - e0 > FIRST ? e0 + FIRST : e1, budget, 0, 0, nullptr, &descents) >= 0) {
+        int lo, span, allowed;
+        strip_bounds(col, lane_rp, e0, &lo, &span, &allowed);
+        if (span > STRIP_BM_WORDS * 32) {
+            // too wide for the bitmap: scan without it, then merge the 16 rows in the first
+            // 16 lanes if the strip is still a candidate
+            const int64_t ch = strip_scan<false>(col, e0, e1, budget, 0, 0, nullptr, &descents);
+            if (ch >= 0 && descents == allowed) {
+                int t = 0;
+                if (lane < 16) {
+                    (void)walk_strip(rowptr, col, M, strip, lane, [&](int, int, unsigned int) {
+                        ++t;
+                        return (int64_t)t <= max_tiles;
+                    });
+                }
+                tiles = __builtin_amdgcn_readfirstlane(t);
+            }
+        } else if (span > 0) {
+            const int words = (span + 31) >> 5;
+            for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
+            wave_lds_order();
+            const int64_t ch = strip_scan<true>(col, e0, e1, budget, lo, span, bm, &descents);
+            wave_lds_order();
+            if (ch >= 0 && descents == allowed) {
+                int t = 0;
+                for (int w = lane; w < words; w += WAVE) t += __builtin_popcount(bm[w]);
+                tiles = wave_sum_i32(t);
+            }
+        }
+        take = tiles > 0 && tiles <= max_tiles && entries >= (int64_t)min_fill * tiles;
+    }
+    if (lane == 0) {
         strip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
         if (take) {
             owner8[2 * strip] = 1;         // both 8-row halves (the array is padded to an even length)
             owner8[2 * strip + 1] = 1;
             spread_add(pc, K_TILES, (unsigned long long)tiles);
-            spread_add(pc, K_NNZ_TILES, (unsigned long long)all_entries);
+            spread_add(pc, K_NNZ_TILES, (unsigned long long)entries);
         }
     }
 }
 
-// pass 2 (after the exclusive scan of strip_ntiles into strip_off): descriptors
-__global__ __launch_bounds__(256) void k_tile_fill(const int32_t *__restrict__ rowptr,
-                                                   const int32_t *__restrict__ col, int M, int64_t n_strips,
-                                                   const unsigned int *__restrict__ strip_ntiles,
-                                                   const unsigned int *__restrict__ strip_off,
-                                                   TileDesc *__restrict__ tiles) {
-    const int64_t strip = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
-    const int sub = threadIdx.x & 15;
+// pass 2 (after the exclusive scan of strip_ntiles into strip_off): strip and tile
+// column of every descriptor, in increasing tile column.  Descriptors of a strip
+// that needs the merging walk are written completely here (pad[0] = 1); the others
+// get their per-row fields from k_tile_rows.
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips,
+    const unsigned int *__restrict__ strip_ntiles, const unsigned int *__restrict__ strip_off,
+    TileDesc *__restrict__ tiles) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
+    const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
     if (strip >= n_strips) return;
     if (strip_ntiles[strip] == 0) return;
-    int64_t at = strip_off[strip];
-    (void)walk_strip(rowptr, col, M, strip, sub, [&](int tj, int first, unsigned int mask) {
-        TileDesc *d = tiles + at;
-        d->off[sub] = first;
-        d->mask[sub] = (uint16_t)mask;
-        if (sub == 0) { d->strip = (int32_t)strip; d->tj = tj; d->pad[0] = 0; d->pad[1] = 0; }
-        ++at;
-        return true;
-    });
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const int64_t r = strip * 16 + lane;
+    const int lane_rp = rowptr[r < M ? r : M];
+    const int e0 = __builtin_amdgcn_readlane(lane_rp, 0), e1 = __builtin_amdgcn_readlane(lane_rp, 16);
+    int lo, span, allowed;
+    strip_bounds(col, lane_rp, e0, &lo, &span, &allowed);
+    const int64_t first_desc = strip_off[strip];
+    if (span > STRIP_BM_WORDS * 32) {
+        if (lane < 16) {
+            int64_t at = first_desc;
+            (void)walk_strip(rowptr, col, M, strip, lane, [&](int tj, int first, unsigned int mask) {
+                TileDesc *d = tiles + at;
+                d->off[lane] = first;
+                d->mask[lane] = (uint16_t)mask;
+                if (lane == 0) { d->strip = (int32_t)strip; d->tj = tj; d->pad[0] = 1; d->pad[1] = 0; }
+                ++at;
+                return true;
+            });
+        }
+        return;
+    }
+    const int words = (span + 31) >> 5;
+    for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
+    wave_lds_order();
+    int64_t descents;
+    (void)strip_scan<true>(col, e0, e1, INT64_MAX, lo, span, bm, &descents);
+    wave_lds_order();
+    int64_t run = first_desc;
+    for (int wb = 0; wb < words; wb += WAVE) {
+        const int w = wb + lane;
+        unsigned int x = w < words ? bm[w] : 0u;
+        const int n = __builtin_popcount(x);
+        int incl = n;
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const int up = __shfl_up(incl, o, WAVE);
+            if (lane >= o) incl += up;
+        }
+        int64_t at = run + (incl - n);
+        while (x) {
+            const int b = __builtin_ctz(x);
+            x &= x - 1;
+            *reinterpret_cast<int4 *>(tiles + at) = make_int4((int)strip, lo + w * 32 + b, 0, 0);
+            ++at;
+        }
+        run += __builtin_amdgcn_readlane(incl, WAVE - 1);
+    }
+}
+
+// pass 3: one thread per (descriptor, row): CSR position of the row's first entry
+// at or after the tile's first column, and the mask of the tile's columns present.
+__global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ rowptr,
+                                                   const int32_t *__restrict__ col, int M,
+                                                   TileDesc *__restrict__ tiles, int64_t n_tiles) {
+    const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t t = slot >> 4;
+    const int sub = (int)(slot & 15);
+    if (t >= n_tiles) return;
+    TileDesc *d = tiles + t;
+    const int4 head = *reinterpret_cast<const int4 *>(d);     // strip, tj, pad[0], pad[1]
+    if (head.z != 0) return;                                   // written by the merging walk
+    const int tj = head.y;
+    const int64_t row = (int64_t)head.x * 16 + sub;
+    int p = 0, end = 0;
+    if (row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
+    const int target = tj * 16;
+    int a = p, b = end;
+    while (a < b) {
+        const int mid = a + ((b - a) >> 1);
+        if (col[mid] < target) a = mid + 1; else b = mid;
+    }
+    unsigned int mask = 0;
+    if (a < end) {
+        const int last = end - 1;
+        int cs[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) cs[j] = col[a + j < last ? a + j : last];
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            if (a + j <= last && (cs[j] >> 4) == tj) mask |= 1u << (cs[j] & 15);
+    }
+    d->off[sub] = a;
+    d->mask[sub] = (uint16_t)mask;
 }
 
 // generic exclusive scan of n unsigned ints: block sums, then apply

@@ -396,9 +396,9 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
         ALLOC_TRY(c, c->d_strip_off, (size_t)n_strips * sizeof(unsigned int));
         c->strips_cap = n_strips;
     }
-    const unsigned walk_grid = (unsigned)((n_strips * 16 + 255) / 256);
-    hipLaunchKernelGGL(k_tile_count, dim3(walk_grid), dim3(256), 0, c->stream, c->d_rowptr, c->d_col, c->sM, n_strips,
-                       min_fill, c->d_strip_ntiles, c->d_owner8, c->d_pc);
+    const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+    hipLaunchKernelGGL(k_strip_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                       c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner8, c->d_pc);
     HIP_TRY(c, hipGetLastError());
     int rc = device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
     if (rc) return rc;
@@ -414,8 +414,11 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
         ALLOC_TRY(c, c->d_tiles, (size_t)c->n_tiles * sizeof(TileDesc));
         c->tiles_cap = c->n_tiles;
     }
-    hipLaunchKernelGGL(k_tile_fill, dim3(walk_grid), dim3(256), 0, c->stream, c->d_rowptr, c->d_col, c->sM, n_strips,
-                       c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
+    hipLaunchKernelGGL(k_strip_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                       c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
+    HIP_TRY(c, hipGetLastError());
+    hipLaunchKernelGGL(k_tile_rows, dim3((unsigned)((c->n_tiles * 16 + 255) / 256)), dim3(256), 0, c->stream,
+                       c->d_rowptr, c->d_col, c->sM, c->d_tiles, c->n_tiles);
     HIP_TRY(c, hipGetLastError());
     c->tiles_active = true;
     c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 4));

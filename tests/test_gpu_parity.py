@@ -411,6 +411,39 @@ def test_tiles_partial_fill_ragged_edges_and_mixed_strips(engine_factory):
     assert st_auto.nnz_mfma >= np.count_nonzero(rows // 16 == 0)
 
 
+def test_tile_strips_wider_than_the_classifier_bitmap(engine_factory):
+    """A strip whose columns span more than 524288 columns does not fit the
+    classifier's per-strip bitmap and is merged row by row instead; strips inside
+    the limit in the same matrix take the bitmap route.  Both must describe the same
+    tiles the host counts."""
+    rng = np.random.default_rng(35)
+    M, N, K = 16 * 5, 700_003, 16
+    r_list, c_list = [], []
+    def block(r0, r1, c0, c1, fill=1.0):
+        m = rng.random((r1 - r0, c1 - c0)) < fill
+        rr, cc = np.nonzero(m)
+        r_list.append(rr + r0); c_list.append(cc + c0)
+    block(0, 16, 0, 48); block(0, 16, N - 40, N)              # strip 0: both ends of a 700k-column span
+    block(16, 32, 1000, 1064, 0.8)                             # strip 1: narrow
+    block(32, 48, 5, 37, 0.9); block(32, 48, 600_000, 600_050, 0.9)   # strip 2: wide, partly filled
+    block(48, 64, 0, N, 0.00002)                               # strip 3: scattered -> gather kernels
+    block(64, 80, 524_288, 524_288 + 16 * 40, 0.7)             # strip 4: narrow span far from column 0
+    r = np.concatenate(r_list).astype(np.int32); c = np.concatenate(c_list).astype(np.int32)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r, c, v)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    rows = np.repeat(np.arange(M), np.diff(rowptr))
+    got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.MFMA_TILE)
+    assert_parity(got, rowptr, col, val, A, B, what="wide strips, forced")
+    assert st.mfma_tiles == _tile_count(rowptr, col, M) and st.nnz_mfma == len(col)
+    got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.AUTO)
+    assert_parity(got, rowptr, col, val, A, B, what="wide strips, auto")
+    keep = rows // 16 != 3
+    assert st.nnz_mfma == np.count_nonzero(keep)
+    assert st.mfma_tiles == _tile_count(rowptr, col, M) - len(np.unique(col[~keep] // 16))
+
+
 def test_tile_path_not_applicable_falls_back_to_gather(engine_factory):
     # K*4 not a multiple of 64 bytes, and bf16 with K=8: everything on the gather kernels
     rng = np.random.default_rng(34)
