@@ -415,11 +415,14 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // One wavefront computes `tiles_per_wave` consecutive tiles.  Operand layout of
 // both MFMA shapes used: lane l supplies row (l & 15) of its operand and the k
 // positions selected by (l >> 4); the result register i of lane l is row
-// 4*(l >> 4) + i, column (l & 15).  A and B are read in 16-byte units: in load
-// step s lane l reads unit 4*s + (l >> 4) of its row, so the four lane groups
-// cover 64 contiguous bytes of each of 16 rows per instruction; which k positions
-// end up in which MFMA does not matter as long as A and B agree.
-// STEPS = row bytes / 64.
+// 4*(l >> 4) + i, column (l & 15).  In step s operand lane l holds the 16-byte unit
+// 4*s + (l >> 4) of its row; which k positions end up in which MFMA does not matter
+// as long as A and B agree.  STEPS = row bytes / 64.
+// The units are READ in another layout -- four neighbouring lanes on the 64
+// contiguous bytes of one row, 16 line segments per instruction instead of the 64 a
+// load in operand layout touches -- and moved into the operand layout through the
+// LDS crossbar (ds_bpermute): the vector memory pipeline pays per line segment that
+// neighbouring lanes touch, not per byte.
 //
 // Software pipeline, three tiles deep, every load unconditional so that the wait
 // counts stay exact (loads return in issue order):
@@ -442,11 +445,21 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
     t_end = t_end < n_tiles ? t_end : n_tiles;
     const int64_t t_last = t_end - 1;
     const int lane = lane_id();
-    const int r16 = lane & 15, q = lane >> 4;
+    const int r16 = lane & 15, q = lane >> 4;        // operand / result layout
+    const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: four neighbouring lanes on 64 bytes of a row
+    const int to_operand_from = (4 * r16 + q) << 2;  // ds_bpermute address: operand lane (r16,q) <- memory lane 4*r16+q
     constexpr uint32_t ROW_UNITS = STEPS * 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     const unsigned int below = (1u << r16) - 1u;
+    auto to_operand = [&](const uint4 &v) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.w);
+        return r;
+    };
 
     struct Desc {
         int strip, tj;
@@ -471,9 +484,9 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
     };
     auto load_oper = [&](const Desc &d) {
         Oper o;
-        int64_t brow = (int64_t)d.tj * 16 + r16;
+        int64_t brow = (int64_t)d.tj * 16 + lrow;
         brow = brow < N ? brow : N - 1;   // columns past N are never in a mask
-        const uint4 *src = Bu + brow * ROW_UNITS + q;
+        const uint4 *src = Bu + brow * ROW_UNITS + lunit;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
         const int offs[4] = {d.off.x, d.off.y, d.off.z, d.off.w};
@@ -499,29 +512,30 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
         const int strip = __builtin_amdgcn_readfirstlane(d_cur.strip);
         if (strip != cur_strip) {
             cur_strip = strip;
-            int64_t arow = (int64_t)strip * 16 + r16;
+            int64_t arow = (int64_t)strip * 16 + lrow;
             arow = arow < M ? arow : M - 1;   // rows past M are never in a mask
-            const uint4 *src = Au + arow * ROW_UNITS + q;
+            const uint4 *src = Au + arow * ROW_UNITS + lunit;
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
+            for (int s = 0; s < STEPS; ++s) a[s] = to_operand(src[s * 4]);
         }
         const Oper o_nxt = load_oper(d_nxt);
         const Desc d_nn = load_desc(t + 2);
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
+            const uint4 b = to_operand(o_cur.b[s]);
             if constexpr (BF16) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
-                                                              __builtin_bit_cast(bf16x8_t, o_cur.b[s]), acc, 0, 0, 0);
+                                                              __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
             } else {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
-                                                           __builtin_bit_cast(float, o_cur.b[s].x), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, b.x), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].y),
-                                                           __builtin_bit_cast(float, o_cur.b[s].y), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, b.y), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].z),
-                                                           __builtin_bit_cast(float, o_cur.b[s].z), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, b.z), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].w),
-                                                           __builtin_bit_cast(float, o_cur.b[s].w), acc, 0, 0, 0);
+                                                           __builtin_bit_cast(float, b.w), acc, 0, 0, 0);
             }
         }
         // scale by S and scatter: result register i is row 4*q+i, column r16
@@ -544,15 +558,29 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
 // The 16 gathered B rows are the "row" operand (lane l: B row of column l&15,
 // 16-byte unit 4s + (l>>4) in step s), the 8 A rows of the panel the "column"
 // operand, held in registers for the whole item.  Result register i of lane l is
-// D[4*(l>>4)+i][l&15]: four CONSECUTIVE entries of row (l&15), so S values and P
-// move as one 16-byte access per lane (rows start at arbitrary 4-byte offsets;
-// global 16-byte accesses need no more alignment than that).  The column indices
+// D[4*(l>>4)+i][l&15]: four consecutive entries of row (l&15).  The column indices
 // are read once for the 8 rows, each gathered B unit serves 8 rows.
+//
+// The vector memory pipeline spends its time per instruction (address cycles for 64
+// lanes) and per line segment that neighbouring lanes touch (one cache lookup each),
+// not per byte, so memory is accessed in a layout of its own, four neighbouring
+// lanes on 64 contiguous bytes, and values change layout inside the wave through
+// the LDS crossbar (ds_bpermute: no memory traffic):
+//   * B:   load lane l reads gathered row l>>2, unit 4s + (l&3): 16 segments per
+//          instruction instead of the 64 a load in operand layout would touch;
+//          operand lane (n,q) then takes its unit from load lane 4n+q;
+//   * S,P: lane l < 32 reads / writes the four consecutive entries 4(l&3).. of row
+//          l>>2 as one 16-byte access (rows start at arbitrary 4-byte offsets; global
+//          16-byte accesses need no more alignment than that): 8 rows x 64 bytes per
+//          instruction; the accumulator is moved into that layout (lane l takes from
+//          result lane 16(l&3) + (l>>2)) and multiplied by S there.
+//
 // Pipeline: the entries are walked in chunks of 64 = 4 groups of 16 columns.  While
 // chunk c computes, the B units and S values of chunk c+1 are in flight (a group is
 // re-requested as soon as its registers have been consumed) and the column indices
-// of chunk c+2 are being read; every load is unconditional (clamped), so the wait
-// counts stay exact and a group only ever waits for loads issued four groups earlier.
+// of chunk c+2 are being read; every load is issued whatever the position (clamped),
+// so the wait counts stay exact and a group only waits for loads issued four groups
+// earlier.
 struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
 
 template <bool BF16, int STEPS>
@@ -572,11 +600,13 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
     const int end = __builtin_amdgcn_readfirstlane(it.end);
     if (start >= end) return;
     const int lane = lane_id();
-    const int n = lane & 15, q = lane >> 4;
+    const int n = lane & 15, q = lane >> 4;          // operand / result layout
+    const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: row, 16-byte unit inside 64 bytes
+    const int to_operand_from = (4 * n + q) << 2;    // ds_bpermute address: operand lane (n,q) <- memory lane 4n+q
+    const int to_memory_from = (16 * lunit + (lrow & 7)) << 2;   // memory lane l <- result lane (row l>>2, q = l&3)
     constexpr int ROW_UNITS = STEPS * 4;
-    // groups of 16 columns in flight; 1, 2 and 4 measured the same (47-50 us on the
-    // FEM shape at K=32): the kernel is not bound by its own prefetch depth
-    constexpr int GROUPS = 4;
+    // groups of 16 columns in flight; 1 KiB rows leave registers for two
+    constexpr int GROUPS = STEPS >= 16 ? 2 : 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored
@@ -589,7 +619,8 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
     // the 8 rows of a panel have one length and follow each other in the CSR arrays
     const int rs0 = __builtin_amdgcn_readfirstlane(it.pad);
     const int row_len = __builtin_amdgcn_readfirstlane(rowptr[row0 + 1]) - rs0;
-    const int64_t out_row = (int64_t)rs0 + (int64_t)(n & 7) * row_len;   // this lane's output row starts here
+    const bool mover = lane < 32;                    // lanes that read S and write P: rows 0..7
+    const int64_t out_row = (int64_t)rs0 + (int64_t)(lrow & 7) * row_len;   // this lane's S/P row starts here
     const int last = end - 1;
     auto cols_of_chunk = [&](int base) {                        // column of entry base + lane (clamped)
         const int e = base + lane < last ? base + lane : last;
@@ -599,66 +630,93 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
         uint4 b[STEPS];
         F4u s;
     };
-    auto load_oper = [&](int c, int g0) {
+    auto load_oper = [&](int cc, int u, int g0) {               // group u of the chunk whose columns are in cc
         Oper o;
-        const uint4 *src = Bu + (int64_t)c * ROW_UNITS + q;
+        const int c = __shfl(cc, u * 16 + lrow, WAVE);
+        const uint4 *src = Bu + (int64_t)c * ROW_UNITS + lunit;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
-        // S values of entries g0+4q .. g0+4q+3 of this lane's row.  The window is clamped
+        // S values of entries g0+4*lunit .. +3 of this lane's row.  The window is clamped
         // into the row (rows of a panel hold at least 4 entries); a clamped window is
         // only ever read for the tail group, which fetches its S values again.
-        const int e = g0 + 4 * q < row_len - 4 ? g0 + 4 * q : row_len - 4;
-        o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
+        const int e = g0 + 4 * lunit < row_len - 4 ? g0 + 4 * lunit : row_len - 4;
+        o.s = F4u{0.f, 0.f, 0.f, 0.f};
+        if (mover) o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
         return o;
+    };
+    auto permute4 = [&](int from, uint32_t x, uint32_t y, uint32_t z, uint32_t w_) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)w_);
+        return r;
     };
     auto compute_store = [&](const Oper &o, int g0) {
         if (g0 >= end) return;                                   // wave-uniform
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
+            const uint4 b = permute4(to_operand_from, o.b[s].x, o.b[s].y, o.b[s].z, o.b[s].w);
             if constexpr (BF16) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, o.b[s]),
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b),
                                                               __builtin_bit_cast(bf16x8_t, a[s]), acc, 0, 0, 0);
             } else {
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].x),
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.x),
                                                            __builtin_bit_cast(float, a[s].x), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].y),
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.y),
                                                            __builtin_bit_cast(float, a[s].y), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].z),
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.z),
                                                            __builtin_bit_cast(float, a[s].z), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, o.b[s].w),
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.w),
                                                            __builtin_bit_cast(float, a[s].w), acc, 0, 0, 0);
             }
         }
-        if (n < 8) {
-            const int e = g0 + 4 * q;
+        // result lane (n,q) holds entries g0+4q.. of row n; memory lane l wants row l>>2,
+        // entries g0+4(l&3)..
+        // (element values first: a bit cast applied to a vector element expression reads element 0)
+        const float r0 = acc[0], r1 = acc[1], r2 = acc[2], r3 = acc[3];
+        const uint4 m = permute4(to_memory_from, __builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1),
+                                 __builtin_bit_cast(uint32_t, r2), __builtin_bit_cast(uint32_t, r3));
+        const float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
+        const float d2 = __builtin_bit_cast(float, m.z), d3 = __builtin_bit_cast(float, m.w);
+        if (mover) {
+            const int e = g0 + 4 * lunit;
             if (g0 + 16 <= end) {
                 // full group: four consecutive entries per lane
-                F4u out{acc[0] * o.s.x, acc[1] * o.s.y, acc[2] * o.s.z, acc[3] * o.s.w};
+                F4u out{d0 * o.s.x, d1 * o.s.y, d2 * o.s.z, d3 * o.s.w};
                 *reinterpret_cast<F4u *>(P + out_row + e) = out;
             } else {
                 // tail group: the S values were read from a clamped window, fetch them again
+                const float d[4] = {d0, d1, d2, d3};
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    if (e + i < end) P[out_row + e + i] = acc[i] * sval[out_row + e + i];
+                    if (e + i < end) P[out_row + e + i] = d[i] * sval[out_row + e + i];
             }
         }
     };
 
     constexpr int CHUNK = GROUPS * 16;                          // columns per loop iteration (<= 64)
     Oper o[GROUPS];
-    {
-        const int cc0 = cols_of_chunk(start);
-#pragma unroll
-        for (int u = 0; u < GROUPS; ++u) o[u] = load_oper(__shfl(cc0, u * 16 + n, WAVE), start + 16 * u);
-    }
+    // Loads complete in issue order and a wait names how many of the most recent ones
+    // may still be in flight.  The waits inside the loop must hold on the way in from
+    // this prologue too, so the prologue issues its loads in the order the loop does
+    // (both column loads first, then the groups in the order they are consumed);
+    // otherwise the loop would wait for almost everything it has just requested.
+    const int cc0 = cols_of_chunk(start);
     int cc_nxt = cols_of_chunk(start + CHUNK);                  // columns of the next chunk
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < GROUPS; ++u) {
+        o[u] = load_oper(cc0, u, start + 16 * u);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     for (int base = start; base < end; base += CHUNK) {
         const int cc_nn = cols_of_chunk(base + 2 * CHUNK);
 #pragma unroll
         for (int u = 0; u < GROUPS; ++u) {
             compute_store(o[u], base + 16 * u);
-            o[u] = load_oper(__shfl(cc_nxt, u * 16 + n, WAVE), base + CHUNK + 16 * u);
+            o[u] = load_oper(cc_nxt, u, base + CHUNK + 16 * u);
         }
         cc_nxt = cc_nn;
     }
