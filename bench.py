@@ -147,9 +147,15 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
-    # ---- per-launch device time from HIP events on the launch stream -----------
+    # ---- device time from HIP events on the launch stream ------------------------
+    # average launch duration: the same K steps between one pair of events (best of 3
+    # regions; what a kernel trace of this loop reports per launch); `isolated` is
+    # each launch between its own events with a wait in between, i.e. with the idle
+    # gap and cold start a lone launch pays
+    region = min(e.time_region(args.steps, include_plan=args.include_plan) for _ in range(3))
+    ev_avg = region / args.steps
     ev = e.time_runs(2, max(args.steps, 20), include_plan=args.include_plan)
-    ev_avg, ev_p50, ev_min = float(ev.mean()), float(np.median(ev)), float(ev.min())
+    ev_p50, ev_min = float(np.median(ev)), float(ev.min())
     # classifier + run in one timed region, for the record (the classifier belongs to
     # the init phase, as the reference's preprocessing does: benchmark.hpp:148-190
     # times init_csr apart from run_csr)
@@ -177,7 +183,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": load_traffic("%s_K%d_%s" % (w.name, w.K, "bf16" if bf16 else "f32"))},
-        "kernel_ms": {"avg": ev_avg, "p50": ev_p50, "min": ev_min, "launches_per_step": st.kernels_launched or 1},
+        "kernel_ms": {"avg": ev_avg, "isolated_p50": ev_p50, "isolated_min": ev_min,
+                      "launches_per_step": st.kernels_launched or 1},
         "gflops_kernel": flops / (ev_avg * 1e-3) / 1e9,
         "bytes_gathered": gathered,
         "bytes_compulsory": w.bytes_compulsory(),

@@ -24,7 +24,7 @@ EXPORTS = [
     "sddmm_create", "sddmm_destroy", "sddmm_strerror", "sddmm_last_error",
     "sddmm_set_dense", "sddmm_set_dense_device", "sddmm_set_csr", "sddmm_set_coo",
     "sddmm_set_csr_device", "sddmm_update_values", "sddmm_plan", "sddmm_run",
-    "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_get_values",
+    "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_get_values",
     "sddmm_get_values_device", "sddmm_last_stats", "sddmm_partition_rows", "sddmm_version",
 ]
 
@@ -86,6 +86,7 @@ def load_library():
     L.sddmm_launch.argtypes = [vp]
     L.sddmm_synchronize.argtypes = [vp]
     L.sddmm_time_runs.argtypes = [vp, i32, i32, i32, vp]
+    L.sddmm_time_region.argtypes = [vp, i32, i32, C.POINTER(C.c_float)]
     L.sddmm_get_values.argtypes = [vp, vp]
     L.sddmm_get_values_device.argtypes = [vp, C.POINTER(vp)]
     L.sddmm_last_stats.argtypes = [vp, C.POINTER(Stats)]
@@ -200,6 +201,12 @@ class Engine:
         ms = np.zeros(max(reps, 1), np.float32)
         self._chk(self.L.sddmm_time_runs(self.h, warmup, reps, int(include_plan), _ptr(ms)))
         return ms[:reps]
+
+    def time_region(self, reps, include_plan=False):
+        """Device milliseconds of `reps` launches back to back between one pair of events."""
+        total = C.c_float(0.0)
+        self._chk(self.L.sddmm_time_region(self.h, reps, int(include_plan), C.byref(total)))
+        return float(total.value)
 
     def values(self):
         P = np.empty(self.nnz, np.float32)

@@ -605,8 +605,8 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
     const int to_operand_from = (4 * n + q) << 2;    // ds_bpermute address: operand lane (n,q) <- memory lane 4n+q
     const int to_memory_from = (16 * lunit + (lrow & 7)) << 2;   // memory lane l <- result lane (row l>>2, q = l&3)
     constexpr int ROW_UNITS = STEPS * 4;
-    // groups of 16 columns in flight; 1 KiB rows leave registers for two
-    constexpr int GROUPS = STEPS >= 16 ? 2 : 4;
+    // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
+    constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored

@@ -1003,6 +1003,34 @@ int sddmm_time_runs(sddmm_ctx *c, int warmup, int reps, int include_plan, float 
     return SDDMM_OK;
 }
 
+int sddmm_time_region(sddmm_ctx *c, int reps, int include_plan, float *total_ms) {
+    if (!c) return SDDMM_ERR_NULL;
+    if (reps < 1) return fail(c, SDDMM_ERR_INVALID, "repetition count must be positive");
+    if (!total_ms) return fail(c, SDDMM_ERR_NULL, "total_ms is NULL");
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    if (!c->planned) {
+        rc = sddmm_plan(c, SDDMM_AUTO);
+        if (rc) return rc;
+    }
+    const int requested = c->requested;
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
+    for (int i = 0; i < reps; ++i) {
+        if (include_plan) {
+            rc = do_plan(c, requested);
+            if (rc) return rc;
+        }
+        rc = enqueue_run(c);
+        if (rc) return rc;
+    }
+    HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
+    HIP_TRY(c, hipEventSynchronize(c->ev1));
+    HIP_TRY(c, hipEventElapsedTime(total_ms, c->ev0, c->ev1));
+    return SDDMM_OK;
+}
+
 int sddmm_get_values(sddmm_ctx *c, float *P_values) {
     if (!c) return SDDMM_ERR_NULL;
     HIP_TRY(c, hipSetDevice(c->device));

@@ -146,6 +146,11 @@ int sddmm_synchronize(sddmm_ctx *ctx);
  * context's stream; ms_each[reps] receives device milliseconds per launch.
  * include_plan != 0 re-runs the classifier inside every timed region. */
 int sddmm_time_runs(sddmm_ctx *ctx, int warmup, int reps, int include_plan, float *ms_each);
+/* reps launches back to back between ONE pair of HIP events on the context's stream:
+ * *total_ms / reps is the average duration of a launch inside a stream of launches
+ * (what a kernel trace of the same loop reports), without the idle gap that the
+ * per-launch synchronisation of sddmm_time_runs puts in front of every launch. */
+int sddmm_time_region(sddmm_ctx *ctx, int reps, int include_plan, float *total_ms);
 
 /* ---- results (cleanup phase) -------------------------------------------- */
 /* nnz floats in the entry order of the input (pattern is never permuted). */

@@ -281,6 +281,27 @@ def test_context_reuse_and_update_values(engine_factory):
     e.close()
 
 
+def test_timing_entry_points(engine_factory):
+    """Per-launch events and one event pair around a stream of launches: both leave
+    the result intact, both report positive times, and a launch inside a stream is
+    not slower than a launch that has to start from an idle device."""
+    rng = np.random.default_rng(13)
+    rowptr, col, val, A, B = _random_case(rng, 600, 500, 32, 0.2)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(600, 500, rowptr, col, val)
+    e.plan(capi.AUTO)
+    each = e.time_runs(2, 20)
+    assert each.shape == (20,) and (each > 0).all()
+    total = min(e.time_region(20) for _ in range(3))
+    assert 0 < total / 20 <= float(np.median(each)) * 1.5
+    assert e.time_region(3, include_plan=True) > 0
+    assert_parity(e.values(), rowptr, col, val, A, B)
+    with pytest.raises(capi.SddmmError):
+        e.time_region(0)
+    e.close()
+
+
 @pytest.mark.parametrize("name", ["small_uniform", "fem_banded", "power_law", "mixed_density"])
 def test_benchmark_shapes_scaled_down(engine_factory, name):
     w = W.make(name, "small")
