@@ -93,3 +93,88 @@ def test_structured_random(engine_factory, seed):
             ok, worst, i = O.check_values(e.values(), refb, mag=magb)
             assert ok, (seed, "bf16", capi.STRATEGY_NAMES[strategy], i, worst)
     e.close()
+
+
+def _host_tile_model(M, rowptr, col, min_fill):
+    """What the strip classifier must decide: a 16-row strip goes to the tile path iff
+    every row is strictly increasing and it holds at least min_fill entries per
+    non-empty 16x16 tile on average."""
+    tiles = entries = 0
+    for s in range((M + 15) // 16):
+        lo, hi = rowptr[s * 16], rowptr[min(M, s * 16 + 16)]
+        if hi == lo:
+            continue
+        ok = True
+        tset = set()
+        for r in range(s * 16, min(M, s * 16 + 16)):
+            c = col[rowptr[r]:rowptr[r + 1]].astype(np.int64)
+            if len(c) > 1 and (np.diff(c) <= 0).any():
+                ok = False
+                break
+            tset.update((c >> 4).tolist())
+        if ok and (hi - lo) >= min_fill * len(tset):
+            tiles += len(tset)
+            entries += hi - lo
+    return tiles, entries
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_strip_classifier_matches_host_model(engine_factory, seed):
+    """Tile counts and covered entries reported by the device classifier against the
+    host model, on matrices whose strips mix clustered, scattered, unsorted and
+    duplicated rows (K=16: 64-byte rows, so the tile path applies)."""
+    rng = np.random.default_rng(7000 + seed)
+    N = int(rng.choice([100, 1000, 40000, 600_000]))
+    M = int(rng.integers(17, 400))
+    rows = []
+    for r in range(M):
+        kind = rng.integers(0, 6)
+        if kind == 0:
+            c = np.zeros(0, np.int64)
+        elif kind == 1:                                   # clustered around a few tile columns
+            base = rng.choice(max(1, N // 16), int(rng.integers(1, 6))) * 16
+            c = np.unique(np.clip((base[:, None] + np.arange(16)[None, :]).ravel(), 0, N - 1))
+            c = c[rng.random(len(c)) < rng.choice([1.0, 0.6])]
+        elif kind == 2:                                   # scattered
+            c = np.sort(rng.choice(N, int(rng.integers(1, min(N, 60))), replace=False))
+        elif kind == 3:                                   # long clustered run
+            s0 = int(rng.integers(0, max(1, N - 700)))
+            c = np.arange(s0, min(N, s0 + int(rng.integers(100, 700))))
+        elif kind == 4 and rng.random() < 0.3:            # not sorted
+            c = rng.permutation(np.sort(rng.choice(N, int(rng.integers(2, min(N, 30))), replace=False)))
+        elif kind == 5 and rng.random() < 0.3:            # a duplicate
+            c = np.sort(rng.choice(N, int(rng.integers(2, min(N, 30))), replace=False))
+            c[1] = c[0]
+        else:
+            c = np.sort(rng.choice(N, int(rng.integers(1, min(N, 20))), replace=False))
+        rows.append(c.astype(np.int64))
+    # make some strips homogeneous so that whole strips qualify
+    for s in range(0, M - 16, 48):
+        base = rng.choice(max(1, N // 16), 3) * 16
+        c = np.unique(np.clip((base[:, None] + np.arange(16)[None, :]).ravel(), 0, N - 1))
+        for r in range(s, s + 16):
+            rows[r] = c[rng.random(len(c)) < 0.8]
+    lens = np.array([len(r) for r in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    K = 16
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    ref = O.sddmm_csr(rowptr, col, val, A, B)
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    for strategy, min_fill in ((capi.MFMA_TILE, 1), (capi.AUTO, 96)):
+        e.plan(strategy)
+        e.run()
+        st = e.stats()
+        want_tiles, want_entries = _host_tile_model(M, rowptr, col, min_fill)
+        if st.strategy_used != capi.FLAT:                 # AUTO may resolve to FLAT when nothing qualifies
+            assert (st.mfma_tiles, st.nnz_mfma) == (want_tiles, want_entries), (seed, capi.STRATEGY_NAMES[strategy], N, M)
+        else:
+            assert want_tiles == 0
+        ok, worst, i = O.check_values(e.values(), ref, mag=mag)
+        assert ok, (seed, capi.STRATEGY_NAMES[strategy], i, worst)
+    e.close()
