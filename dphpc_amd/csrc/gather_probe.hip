@@ -1,0 +1,74 @@
+// Row-gather yardstick: n rows of 128 bytes, picked at random from a table of T
+// rows, read with 8 neighbouring lanes x 16 bytes per row and 8 rows in flight per
+// lane -- the access pattern of the SDDMM gather kernels with everything else
+// (A rows, indices, S values, FMAs, P stores) taken away.  What it reaches is the
+// ceiling of the box for that pattern at a given table size (L2-resident,
+// last-level-cache-resident, HBM).
+// usage: gather_probe [n rows] [table rows] [blocks] [sequential 0|1]
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+#define CHECK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_)); return 1; } } while (0)
+
+__global__ __launch_bounds__(256) void gather_probe_kernel(const uint4 *__restrict__ table, const int *__restrict__ idx,
+                                                           long n, unsigned *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const int g = lane >> 3, j = lane & 7;
+    unsigned acc = 0;
+    // chunks of 64 rows per wave: lane l reads the index of row l, then 8 steps of 8 rows
+    for (long base = wave * 64; base < n; base += nwaves * 64) {
+        const int mine = idx[base + lane < n ? base + lane : n - 1];
+        uint4 v[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int r = __shfl(mine, s * 8 + g, 64);
+            v[s] = table[(long)r * 8 + j];
+        }
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc ^= v[s].x ^ v[s].y ^ v[s].z ^ v[s].w;
+    }
+    if (acc == 0x12345678u) out[0] = acc;   // keeps the loads alive
+}
+
+int main(int argc, char **argv) {
+    const long n = argc > 1 ? atol(argv[1]) : 2000000;
+    const long T = argc > 2 ? atol(argv[2]) : 30000;
+    const int blocks = argc > 3 ? atoi(argv[3]) : 2048;
+    const int seq = argc > 4 ? atoi(argv[4]) : 0;
+    if (n < 1 || T < 1 || T > 2147483647L || blocks < 1) { fprintf(stderr, "bad arguments\n"); return 2; }
+    std::vector<int> h((size_t)n);
+    std::mt19937_64 rng(1);
+    for (long i = 0; i < n; ++i) h[(size_t)i] = seq ? (int)(i % T) : (int)(rng() % (unsigned long)T);
+    uint4 *table = nullptr;
+    int *idx = nullptr;
+    unsigned *out = nullptr;
+    CHECK(hipMalloc((void **)&table, (size_t)T * 128));
+    CHECK(hipMemset(table, 1, (size_t)T * 128));
+    CHECK(hipMalloc((void **)&idx, (size_t)n * 4));
+    CHECK(hipMemcpy(idx, h.data(), (size_t)n * 4, hipMemcpyHostToDevice));
+    CHECK(hipMalloc((void **)&out, 4));
+    hipEvent_t a, b;
+    CHECK(hipEventCreate(&a));
+    CHECK(hipEventCreate(&b));
+    for (int w = 0; w < 3; ++w) hipLaunchKernelGGL(gather_probe_kernel, dim3(blocks), dim3(256), 0, 0, table, idx, n, out);
+    CHECK(hipDeviceSynchronize());
+    const int reps = 20;
+    CHECK(hipEventRecord(a, 0));
+    for (int r = 0; r < reps; ++r) hipLaunchKernelGGL(gather_probe_kernel, dim3(blocks), dim3(256), 0, 0, table, idx, n, out);
+    CHECK(hipEventRecord(b, 0));
+    CHECK(hipEventSynchronize(b));
+    float ms = 0.f;
+    CHECK(hipEventElapsedTime(&ms, a, b));
+    const double us = ms * 1e3 / reps;
+    printf("rows=%ld table=%ld rows (%.1f MB) blocks=%d %s: %.1f us per launch, %.1f G rows/s, %.2f TB/s gathered\n", n, T,
+           T * 128 / 1e6, blocks, seq ? "sequential" : "random", us, n / us / 1e3, n * 128.0 / us / 1e6);
+    CHECK(hipFree(table));
+    CHECK(hipFree(idx));
+    CHECK(hipFree(out));
+    return 0;
+}
