@@ -90,6 +90,7 @@ def main():
     ap.add_argument("--K", type=int, default=32)
     ap.add_argument("--strategy", default="AUTO")
     ap.add_argument("--include-plan", action="store_true", help="re-run the classifier inside every timed step")
+    ap.add_argument("--f16", action="store_true", help="dense_tiles: IEEE half operands instead of bf16")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip validation against the oracle")
     args = ap.parse_args()
@@ -103,14 +104,15 @@ def main():
     from dphpc_amd import capi, workloads
 
     t0 = time.time()
-    w = workloads.make(args.workload, args.size, K=args.K)
+    extra = {"f16": True} if args.f16 and args.workload == "dense_tiles" else {}
+    w = workloads.make(args.workload, args.size, K=args.K, **extra)
     log("workload %s: M=%d N=%d K=%d nnz=%d (%.1fs to generate)" % (w.name, w.M, w.N, w.K, w.nnz, time.time() - t0))
     strategy = capi.STRATEGY_NAMES.index(args.strategy.upper())
-    bf16 = w.dtype == "bf16"
+    bf16 = w.dtype != "f32"          # 16-bit operands (bf16 or IEEE half)
 
     e = capi.Engine(0)
     if bf16:
-        e.set_dense(w.A_bits, w.B_bits, capi.BF16)
+        e.set_dense(w.A_bits, w.B_bits, capi.BF16 if w.dtype == "bf16" else capi.F16)
     else:
         e.set_dense(w.A, w.B, capi.F32)
     e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
@@ -175,14 +177,14 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if bf16 else "f32",
+        "dtype": w.dtype,
         "data": "synthetic",
         "config": {"workload": w.name, "size": args.size, "M": w.M, "N": w.N, "K": w.K, "nnz": w.nnz,
                    "strategy": capi.STRATEGY_NAMES[st.strategy_used], "requested": args.strategy.upper(),
                    "plan_in_step": bool(args.include_plan)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": load_traffic("%s_K%d_%s" % (w.name, w.K, "bf16" if bf16 else "f32"))},
+                     "traffic": load_traffic("%s_K%d_%s" % (w.name, w.K, w.dtype))},
         "kernel_ms": {"avg": ev_avg, "isolated_p50": ev_p50, "isolated_min": ev_min,
                       "launches_per_step": st.kernels_launched or 1},
         "gflops_kernel": flops / (ev_avg * 1e-3) / 1e9,

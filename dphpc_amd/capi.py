@@ -14,7 +14,7 @@ _LIB_PATH = os.environ.get("SDDMM_LIB") or os.path.join(_PKG, "lib", "libsddmm_a
 
 AUTO, FLAT, ROW_WAVE, SHORT_ROWS, LDS_TILED, MFMA_TILE, EXACT = range(7)
 STRATEGY_NAMES = ["AUTO", "FLAT", "ROW_WAVE", "SHORT_ROWS", "LDS_TILED", "MFMA_TILE", "EXACT"]
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 
 OK, ERR_INVALID, ERR_NULL, ERR_STATE, ERR_ALLOC, ERR_HIP, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_PATTERN = (
     0, -1, -2, -3, -4, -5, -6, -7, -8)
@@ -109,6 +109,15 @@ def to_bf16(x):
 
 def from_bf16(b):
     return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def to_f16(x):
+    """fp32 -> IEEE half bit patterns (uint16), round to nearest even."""
+    return np.ascontiguousarray(x, np.float32).astype(np.float16).view(np.uint16)
+
+
+def from_f16(b):
+    return np.ascontiguousarray(b, np.uint16).view(np.float16).astype(np.float32)
 
 
 def partition_rows(rowptr, parts, stride=1):

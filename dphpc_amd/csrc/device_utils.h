@@ -93,7 +93,7 @@ struct RowItem {
 
 // ---- units of the K dimension ----------------------------------------------
 // A "unit" is what one lane loads per step along K: 16 bytes where alignment
-// allows (4 fp32 or 8 bf16), one fp32 otherwise.  dot() extends an fp32
+// allows (4 fp32, 8 bf16 or 8 fp16), one fp32 otherwise.  dot() extends an fp32
 // accumulator with fused multiply-adds in element order.
 struct UnitF32x4 {
     using T = float4;
@@ -133,5 +133,27 @@ struct UnitBF16x8 {
         return acc;
     }
 };
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+struct UnitF16x8 {
+    using T = uint4;  // 8 IEEE half floats, two per 32-bit word, low half first
+    static constexpr int ELEMS = 8;
+    static __device__ __forceinline__ T zero() { return make_uint4(0u, 0u, 0u, 0u); }
+    // v_dot2c_f32_f16: acc + a.lo*b.lo + a.hi*b.hi with fp32 accumulation (products of
+    // halves are exact in fp32)
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), acc, false);
+    }
+    static __device__ __forceinline__ float dot(const T &a, const T &b, float acc) {
+        acc = dot2(a.x, b.x, acc);
+        acc = dot2(a.y, b.y, acc);
+        acc = dot2(a.z, b.z, acc);
+        acc = dot2(a.w, b.w, acc);
+        return acc;
+    }
+};
+
+// element types of A and B as template arguments of the kernels
+constexpr int DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2;
 
 }  // namespace sddmm

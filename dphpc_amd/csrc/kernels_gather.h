@@ -571,7 +571,7 @@ __global__ __launch_bounds__(BLOCK, SDDMM_PANEL_OCC) void k_panel(const void *__
 // EXACT: one lane per entry, k ascending, separate fp32 multiply and add (the
 // translation unit is compiled with -ffp-contract=off), then the multiply by S:
 // the operation sequence of the CPU loop, hence bit-identical to it.
-template <bool IS_BF16>
+template <int DT>
 __global__ __launch_bounds__(BLOCK) void k_exact(const void *__restrict__ Av, const void *__restrict__ Bv,
                                                  int K, const int32_t *__restrict__ rowidx,
                                                  const int32_t *__restrict__ col,
@@ -581,12 +581,20 @@ __global__ __launch_bounds__(BLOCK) void k_exact(const void *__restrict__ Av, co
     if (n >= nnz) return;
     const int64_t r = rowidx[n], c = col[n];
     float acc = 0.f;
-    if constexpr (IS_BF16) {
+    if constexpr (DT == DT_BF16) {
         const uint16_t *a = (const uint16_t *)Av + r * K;
         const uint16_t *b = (const uint16_t *)Bv + c * K;
         for (int k = 0; k < K; ++k) {
             const float x = __builtin_bit_cast(float, (uint32_t)a[k] << 16);
             const float y = __builtin_bit_cast(float, (uint32_t)b[k] << 16);
+            const float prod = x * y;
+            acc = acc + prod;
+        }
+    } else if constexpr (DT == DT_F16) {
+        const _Float16 *a = (const _Float16 *)Av + r * K;
+        const _Float16 *b = (const _Float16 *)Bv + c * K;
+        for (int k = 0; k < K; ++k) {
+            const float x = (float)a[k], y = (float)b[k];
             const float prod = x * y;
             acc = acc + prod;
         }

@@ -12,7 +12,7 @@
 //     computed here, sparse tiles included) or not at all, so the gather kernels
 //     and this one never share a row;
 //   * k_tile computes the full 16x16 product A[strip rows] * B[tile cols]^T with
-//     fp32 accumulation (bf16: v_mfma_f32_16x16x32_bf16, fp32: v_mfma_f32_16x16x4_f32,
+//     fp32 accumulation (bf16 / fp16: v_mfma_f32_16x16x32_bf16 / _f16, fp32: v_mfma_f32_16x16x4_f32,
 //     both exact products of the stored inputs), multiplies by the S values and
 //     writes only the positions the masks name -- P keeps S's order.
 //
@@ -410,6 +410,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_apply(const unsigned int *_
 
 // ---- the MFMA kernel ------------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 // One wavefront computes `tiles_per_wave` consecutive tiles.  Operand layout of
@@ -431,7 +432,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //   and then computes    MFMAs of tile t, scale, scatter (operands landed during t-1)
 // The A panel of the current strip stays in registers and is reloaded only when
 // the strip changes (a wave-uniform branch placed before the iteration's loads).
-template <bool BF16, int STEPS>
+template <int DT, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                 int tiles_per_wave, const float *__restrict__ sval,
@@ -524,9 +525,12 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             const uint4 b = to_operand(o_cur.b[s]);
-            if constexpr (BF16) {
+            if constexpr (DT == DT_BF16) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
                                                               __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+            } else if constexpr (DT == DT_F16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a[s]),
+                                                             __builtin_bit_cast(half8_t, b), acc, 0, 0, 0);
             } else {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
                                                            __builtin_bit_cast(float, b.x), acc, 0, 0, 0);
@@ -583,7 +587,7 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
 // earlier.
 struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
 
-template <bool BF16, int STEPS>
+template <int DT, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
@@ -658,9 +662,12 @@ __global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             const uint4 b = permute4(to_operand_from, o.b[s].x, o.b[s].y, o.b[s].z, o.b[s].w);
-            if constexpr (BF16) {
+            if constexpr (DT == DT_BF16) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b),
                                                               __builtin_bit_cast(bf16x8_t, a[s]), acc, 0, 0, 0);
+            } else if constexpr (DT == DT_F16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, b),
+                                                             __builtin_bit_cast(half8_t, a[s]), acc, 0, 0, 0);
             } else {
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.x),
                                                            __builtin_bit_cast(float, a[s].x), acc, 0, 0, 0);

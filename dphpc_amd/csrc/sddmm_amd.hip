@@ -148,7 +148,7 @@ void release_sparse(sddmm_ctx *c) {
     c->nnz = 0;
 }
 
-size_t elem_size(int dtype) { return dtype == SDDMM_BF16 ? 2 : 4; }
+size_t elem_size(int dtype) { return dtype == SDDMM_F32 ? 4 : 2; }
 
 int grid_for(int64_t n, int block) { return (int)std::max<int64_t>(1, (n + block - 1) / block); }
 int grid_capped(int64_t n, int block, int cap = 16384) {
@@ -164,7 +164,7 @@ int fetch_counters(sddmm_ctx *c) {
 
 // ---- kernel dispatch over the (unit type, lanes per entry, units per lane) layouts ----
 struct Shape {
-    int unit;    // 0: fp32 x4, 1: fp32 x1, 2: bf16 x8
+    int unit;    // 0: fp32 x4, 1: fp32 x1, 2: bf16 x8, 3: fp16 x8
     int KU;      // units per row
     int LPN;     // lanes per entry (0: row too long for the register layout)
     int UPL;     // units per lane
@@ -181,7 +181,7 @@ int pow2ceil(int x) {
 Shape shape_of(const sddmm_ctx *c) {
     Shape s{};
     size_t unit_bytes;
-    if (c->dtype == SDDMM_BF16) { s.unit = 2; s.KU = c->K / 8; unit_bytes = 16; }
+    if (c->dtype == SDDMM_BF16 || c->dtype == SDDMM_F16) { s.unit = c->dtype == SDDMM_BF16 ? 2 : 3; s.KU = c->K / 8; unit_bytes = 16; }
     else if (c->K % 4 == 0) { s.unit = 0; s.KU = c->K / 4; unit_bytes = 16; }
     else { s.unit = 1; s.KU = c->K; unit_bytes = 4; }
     if (s.unit == 1) {
@@ -231,6 +231,7 @@ template <class F>
 void with_layout(const Shape &s, F &&f) {
     if (s.unit == 0) with_layout16<UnitF32x4>(s, f);
     else if (s.unit == 2) with_layout16<UnitBF16x8>(s, f);
+    else if (s.unit == 3) with_layout16<UnitF16x8>(s, f);
     else if (s.LPN == 0) f(Layout<UnitF32x1, 0, 1, false, true>{});
     else if (s.LPN == 4) with_mask_width<UnitF32x1, 4, 1>(s, f);
     else if (s.UPL == 1) with_mask_width<UnitF32x1, 16, 1>(s, f);
@@ -428,7 +429,7 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
 // Row-panel detector (8 consecutive rows, 8-aligned, same column list).  Two
 // kernels can run the panels: the MFMA one (row size a multiple of 64 bytes, up to
 // 1 KiB) and the VALU one (8-lanes-per-entry layouts whose 8 A rows fit in
-// registers: fp32 K = 32 or 64, bf16 K = 64, 32-bit offsets); the VALU kernel has
+// registers: fp32 K = 32 or 64, bf16 / fp16 K = 64, 32-bit offsets); the VALU kernel has
 // the per-entry arithmetic of the gather kernels, the MFMA kernel is faster.
 int panel_mfma_steps(const sddmm_ctx *c) {
     const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
@@ -492,56 +493,59 @@ void launch_panel_u(sddmm_ctx *c, const Shape &s) {
     if (s.UPL == 1) launch_panel_t<U, 1>(c, s.KU);
     else launch_panel_t<U, 2>(c, s.KU);
 }
-template <bool BF16, int STEPS>
+template <int DT, int STEPS>
 void launch_panel_mfma_t(sddmm_ctx *c) {
     const int64_t nblocks = (c->n_panel_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_panel_mfma<BF16, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+    hipLaunchKernelGGL((k_panel_mfma<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
                        (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
                        c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
 }
-template <bool BF16>
+template <int DT>
 void launch_panel_mfma_steps(sddmm_ctx *c) {
     switch (panel_mfma_steps(c)) {
-        case 1: launch_panel_mfma_t<BF16, 1>(c); break;
-        case 2: launch_panel_mfma_t<BF16, 2>(c); break;
-        case 4: launch_panel_mfma_t<BF16, 4>(c); break;
-        case 8: launch_panel_mfma_t<BF16, 8>(c); break;
-        default: launch_panel_mfma_t<BF16, 16>(c); break;
+        case 1: launch_panel_mfma_t<DT, 1>(c); break;
+        case 2: launch_panel_mfma_t<DT, 2>(c); break;
+        case 4: launch_panel_mfma_t<DT, 4>(c); break;
+        case 8: launch_panel_mfma_t<DT, 8>(c); break;
+        default: launch_panel_mfma_t<DT, 16>(c); break;
     }
 }
 
 void launch_panels(sddmm_ctx *c) {
     if (c->panel_mfma) {
-        if (c->dtype == SDDMM_BF16) launch_panel_mfma_steps<true>(c);
-        else launch_panel_mfma_steps<false>(c);
+        if (c->dtype == SDDMM_BF16) launch_panel_mfma_steps<DT_BF16>(c);
+        else if (c->dtype == SDDMM_F16) launch_panel_mfma_steps<DT_F16>(c);
+        else launch_panel_mfma_steps<DT_F32>(c);
         return;
     }
     const Shape s = shape_of(c);
     if (s.unit == 0) launch_panel_u<UnitF32x4>(c, s);
-    else launch_panel_t<UnitBF16x8, 1>(c, s.KU);
+    else if (s.unit == 2) launch_panel_t<UnitBF16x8, 1>(c, s.KU);
+    else launch_panel_t<UnitF16x8, 1>(c, s.KU);
 }
 
-template <bool BF16, int STEPS>
+template <int DT, int STEPS>
 void launch_tile_t(sddmm_ctx *c) {
     const int64_t waves = (c->n_tiles + c->tiles_per_wave - 1) / c->tiles_per_wave;
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_tile<BF16, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+    hipLaunchKernelGGL((k_tile<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const TileDesc *)c->d_tiles, c->n_tiles,
                        c->tiles_per_wave, (const float *)c->d_sval, c->dP, nblocks);
 }
-template <bool BF16>
+template <int DT>
 void launch_tile_steps(sddmm_ctx *c) {
     switch (c->tile_steps) {
-        case 1: launch_tile_t<BF16, 1>(c); break;
-        case 2: launch_tile_t<BF16, 2>(c); break;
-        case 4: launch_tile_t<BF16, 4>(c); break;
-        case 8: launch_tile_t<BF16, 8>(c); break;
-        default: launch_tile_t<BF16, 16>(c); break;
+        case 1: launch_tile_t<DT, 1>(c); break;
+        case 2: launch_tile_t<DT, 2>(c); break;
+        case 4: launch_tile_t<DT, 4>(c); break;
+        case 8: launch_tile_t<DT, 8>(c); break;
+        default: launch_tile_t<DT, 16>(c); break;
     }
 }
 void launch_tiles(sddmm_ctx *c) {
-    if (c->dtype == SDDMM_BF16) launch_tile_steps<true>(c);
-    else launch_tile_steps<false>(c);
+    if (c->dtype == SDDMM_BF16) launch_tile_steps<DT_BF16>(c);
+    else if (c->dtype == SDDMM_F16) launch_tile_steps<DT_F16>(c);
+    else launch_tile_steps<DT_F32>(c);
 }
 
 int ensure_rowidx(sddmm_ctx *c) {
@@ -604,10 +608,13 @@ int enqueue_run(sddmm_ctx *c) {
             break;
         case SDDMM_EXACT:
             if (c->dtype == SDDMM_BF16)
-                hipLaunchKernelGGL(k_exact<true>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                hipLaunchKernelGGL(k_exact<DT_BF16>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                                   c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
+            else if (c->dtype == SDDMM_F16)
+                hipLaunchKernelGGL(k_exact<DT_F16>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
                                    c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
             else
-                hipLaunchKernelGGL(k_exact<false>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                hipLaunchKernelGGL(k_exact<DT_F32>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
                                    c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
             break;
         default: return fail(c, SDDMM_ERR_STATE, "no kernel for strategy %d", c->strategy);
@@ -759,8 +766,9 @@ static int set_dense_common(sddmm_ctx *c, int M, int N, int K, const void *A, co
     if (!c) return SDDMM_ERR_NULL;
     HIP_TRY(c, hipSetDevice(c->device));
     if (M < 0 || N < 0 || K < 1) return fail(c, SDDMM_ERR_INVALID, "need M,N >= 0 and K >= 1 (got %d,%d,%d)", M, N, K);
-    if (dtype != SDDMM_F32 && dtype != SDDMM_BF16) return fail(c, SDDMM_ERR_INVALID, "unknown dtype %d", dtype);
-    if (dtype == SDDMM_BF16 && K % 8) return fail(c, SDDMM_ERR_INVALID, "bf16 operands need K %% 8 == 0 (got %d)", K);
+    if (dtype != SDDMM_F32 && dtype != SDDMM_BF16 && dtype != SDDMM_F16)
+        return fail(c, SDDMM_ERR_INVALID, "unknown dtype %d", dtype);
+    if (dtype != SDDMM_F32 && K % 8) return fail(c, SDDMM_ERR_INVALID, "16-bit operands need K %% 8 == 0 (got %d)", K);
     if ((M > 0 && !A) || (N > 0 && !B)) return fail(c, SDDMM_ERR_NULL, "A or B is NULL");
     release_dense(c);
     const size_t es = elem_size(dtype);

@@ -26,8 +26,8 @@ class Workload:
     sval: np.ndarray
     A: np.ndarray                 # fp32 (for bf16 workloads: the bf16-rounded values)
     B: np.ndarray
-    dtype: str = "f32"            # "f32" | "bf16"
-    A_bits: np.ndarray = None     # uint16 bf16 bit patterns when dtype == "bf16"
+    dtype: str = "f32"            # "f32" | "bf16" | "f16"
+    A_bits: np.ndarray = None     # uint16 bit patterns when dtype is "bf16" or "f16"
     B_bits: np.ndarray = None
     meta: dict = field(default_factory=dict)
 
@@ -43,12 +43,12 @@ class Workload:
         return 2.0 * self.nnz * self.K
 
     def bytes_gathered(self):
-        e = 2 if self.dtype == "bf16" else 4
+        e = 4 if self.dtype == "f32" else 2
         nonempty = int(np.count_nonzero(np.diff(self.rowptr)))
         return 4.0 * (self.M + 1) + 12.0 * self.nnz + e * self.K * nonempty + e * self.K * self.nnz
 
     def bytes_compulsory(self):
-        e = 2 if self.dtype == "bf16" else 4
+        e = 4 if self.dtype == "f32" else 2
         nonempty = int(np.count_nonzero(np.diff(self.rowptr)))
         touched = int(len(np.unique(self.col)))
         return 4.0 * (self.M + 1) + 12.0 * self.nnz + e * self.K * (nonempty + touched)
@@ -192,11 +192,11 @@ def mixed_density(K=32, M=30000, dense_frac=0.10, window=1385, fill=0.40, seed=S
 
 
 # --------------------------------------------------------------------------- 5
-def dense_tiles(K=128, M=4562, N=5761, tile_frac=0.09377, seed=SEED_BASE + 5, bf16=True):
+def dense_tiles(K=128, M=4562, N=5761, tile_frac=0.09377, seed=SEED_BASE + 5, bf16=True, f16=False):
     """Fully dense 16x16 tiles at random tile positions; A,B in bf16 (round to
     nearest even of U[-1,1]) with the fp32 view of the rounded values kept for the
-    oracle."""
-    from .capi import to_bf16, from_bf16
+    oracle.  bf16=False: fp32 operands; f16=True: IEEE half instead of bf16."""
+    from .capi import to_bf16, from_bf16, to_f16, from_f16
     rng = np.random.default_rng(seed)
     tr, tc = M // 16, N // 16
     n_tiles = int(round(tr * tc * tile_frac))
@@ -210,6 +210,11 @@ def dense_tiles(K=128, M=4562, N=5761, tile_frac=0.09377, seed=SEED_BASE + 5, bf
     sval = rng.random(len(col), dtype=np.float32)
     A = _dense(rng, M, K, "uniform")
     B = _dense(rng, N, K, "uniform")
+    if f16:
+        Ab, Bb = to_f16(A), to_f16(B)
+        return Workload("dense_tiles", M, N, K, rowptr, col, sval,
+                        from_f16(Ab).reshape(M, K), from_f16(Bb).reshape(N, K), dtype="f16",
+                        A_bits=Ab.reshape(M, K), B_bits=Bb.reshape(N, K), meta={"tiles": n_tiles})
     if not bf16:
         return Workload("dense_tiles", M, N, K, rowptr, col, sval, A, B, meta={"tiles": n_tiles})
     Ab, Bb = to_bf16(A), to_bf16(B)

@@ -49,7 +49,10 @@ enum sddmm_status {
 
 enum sddmm_dtype {
     SDDMM_F32 = 0,  /* A,B fp32; fp32 accumulate                                     */
-    SDDMM_BF16 = 1  /* A,B bfloat16 (uint16 storage); fp32 accumulate and output     */
+    SDDMM_BF16 = 1, /* A,B bfloat16 (uint16 storage); fp32 accumulate and output     */
+    SDDMM_F16 = 2   /* A,B IEEE half (uint16 storage); fp32 accumulate and output --
+                       the input type of the reference's tensor-core sketch,
+                       src/competitors/gpu/gpu_tensor.cu:27-99                       */
 };
 
 /* Kernel selection.  The reference picks between two kernels from one global
@@ -111,7 +114,7 @@ const char *sddmm_last_error(const sddmm_ctx *ctx);
 /* A: M*K elements, B: N*K elements, row-major, leading dimension K
  * (src/matrices/Dense.hpp:43-50).  K >= 1; any K is accepted for SDDMM_F32
  * (the reference's kernels need K%8 or K%32, gpu_basic.cu:77-80, gpu_shared.cu:98-101);
- * SDDMM_BF16 needs K % 8 == 0. */
+ * SDDMM_BF16 and SDDMM_F16 need K % 8 == 0. */
 int sddmm_set_dense(sddmm_ctx *ctx, int M, int N, int K, const void *A, const void *B, int dtype);
 /* Same, A and B already in device memory of this ctx's device (borrowed, 16-byte aligned). */
 int sddmm_set_dense_device(sddmm_ctx *ctx, int M, int N, int K, const void *dA, const void *dB, int dtype);

@@ -325,6 +325,29 @@ def test_bf16_inputs_gather_path(engine_factory, K):
         assert_parity(got, w.rowptr, w.col, w.sval, w.A, w.B, rtol=1e-5, exact=(strategy == capi.EXACT), what="bf16")
 
 
+@pytest.mark.parametrize("K", [8, 32, 128, 512, 1032])
+def test_f16_inputs(engine_factory, K):
+    """IEEE half inputs with fp32 accumulation on every path (gather kernels with
+    v_dot2c_f32_f16, dense tiles on v_mfma_f32_16x16x32_f16).  Products of halves are
+    exact in fp32, so the fp32 bar applies; EXACT is bit-identical to the oracle on
+    the half-rounded inputs."""
+    w = W.make("dense_tiles", "small", K=K, bf16=False)
+    Ab, Bb = capi.to_f16(w.A).reshape(w.M, K), capi.to_f16(w.B).reshape(w.N, K)
+    A, B = capi.from_f16(Ab).reshape(w.M, K), capi.from_f16(Bb).reshape(w.N, K)
+    tiled = (2 * K) % 64 == 0 and 2 * K <= 1024
+    for strategy in (capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.AUTO, capi.MFMA_TILE, capi.EXACT):
+        _say("f16", K, capi.STRATEGY_NAMES[strategy])
+        got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, Ab, Bb, w.N, strategy, capi.F16)
+        assert_parity(got, w.rowptr, w.col, w.sval, A, B, rtol=1e-5, exact=(strategy == capi.EXACT), what="f16 K=%d" % K)
+        if strategy in (capi.AUTO, capi.MFMA_TILE):
+            assert (st.mfma_tiles == w.meta["tiles"]) == tiled and (st.mfma_tiles == 0) == (not tiled)
+    # K must be a multiple of 8 for 16-bit operands
+    e = engine_factory()
+    with pytest.raises(capi.SddmmError):
+        e.set_dense(np.zeros((4, 12), np.uint16), np.zeros((4, 12), np.uint16), capi.F16)
+    e.close()
+
+
 def test_auto_resolves_to_flat_when_short_rows_dominate(engine_factory):
     w = W.make("power_law", "small")
     got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, w.A, w.B, w.N, capi.AUTO)
@@ -496,7 +519,7 @@ def test_fem_blocks_tiles_and_panels(engine_factory, monkeypatch):
 
 
 @pytest.mark.parametrize("K,dtype", [(32, "f32"), (64, "f32"), (128, "f32"), (256, "f32"), (64, "bf16"), (256, "bf16"),
-                                     (24, "f32"), (33, "f32")])
+                                     (24, "f32"), (33, "f32"), (32, "f16"), (64, "f16"), (512, "f16")])
 def test_row_panels(engine_factory, monkeypatch, K, dtype):
     """Groups of identical rows: aligned 8-row panels are taken, everything else
     (unaligned groups, groups of other sizes, rows with one differing column, short
@@ -533,11 +556,15 @@ def test_row_panels(engine_factory, monkeypatch, K, dtype):
         Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
         A, B = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K)
         ops, dt = (Ab, Bb), capi.BF16
+    elif dtype == "f16":
+        Ab, Bb = capi.to_f16(A).reshape(M, K), capi.to_f16(B).reshape(N, K)
+        A, B = capi.from_f16(Ab).reshape(M, K), capi.from_f16(Bb).reshape(N, K)
+        ops, dt = (Ab, Bb), capi.F16
     else:
         ops, dt = (A, B), capi.F32
-    row_bytes = K * (2 if dtype == "bf16" else 4)
+    row_bytes = K * (4 if dtype == "f32" else 2)
     applicable = row_bytes % 64 == 0                                         # the MFMA panel kernel
-    valu_applicable = (dtype, K) in (("f32", 32), ("f32", 64), ("bf16", 64))  # A rows of a panel fit in registers
+    valu_applicable = (dtype, K) in (("f32", 32), ("f32", 64), ("bf16", 64), ("f16", 64))  # A rows of a panel fit in registers
     same = len(rows_cols[51]) == 50 and np.array_equal(rows_cols[51], rows_cols[48])
     assert not same
     for strategy, min_len in ((capi.LDS_TILED, 1), (capi.AUTO, 16)):
