@@ -95,7 +95,11 @@ struct RowItem {
 // A "unit" is what one lane loads per step along K: 16 bytes where alignment
 // allows (4 fp32, 8 bf16 or 8 fp16), one fp32 otherwise.  dot() extends an fp32
 // accumulator with fused multiply-adds in element order.
+// element types of A and B as template arguments of the kernels
+constexpr int DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2;
+
 struct UnitF32x4 {
+    static constexpr int DT = DT_F32;
     using T = float4;
     static constexpr int ELEMS = 4;
     static __device__ __forceinline__ T zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
@@ -108,6 +112,7 @@ struct UnitF32x4 {
     }
 };
 struct UnitF32x1 {
+    static constexpr int DT = DT_F32;
     using T = float;
     static constexpr int ELEMS = 1;
     static __device__ __forceinline__ T zero() { return 0.f; }
@@ -116,6 +121,7 @@ struct UnitF32x1 {
     }
 };
 struct UnitBF16x8 {
+    static constexpr int DT = DT_BF16;
     using T = uint4;  // 8 bfloat16, two per 32-bit word, low half first
     static constexpr int ELEMS = 8;
     static __device__ __forceinline__ T zero() { return make_uint4(0u, 0u, 0u, 0u); }
@@ -136,6 +142,7 @@ struct UnitBF16x8 {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 struct UnitF16x8 {
+    static constexpr int DT = DT_F16;
     using T = uint4;  // 8 IEEE half floats, two per 32-bit word, low half first
     static constexpr int ELEMS = 8;
     static __device__ __forceinline__ T zero() { return make_uint4(0u, 0u, 0u, 0u); }
@@ -152,8 +159,5 @@ struct UnitF16x8 {
         return acc;
     }
 };
-
-// element types of A and B as template arguments of the kernels
-constexpr int DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2;
 
 }  // namespace sddmm

@@ -282,7 +282,7 @@ __device__ __forceinline__ void row_segment_body(const void *__restrict__ A, con
 template <class L>
 __device__ __forceinline__ void short_rows_body(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                 const int32_t *__restrict__ rowptr,
-                                                const unsigned char *__restrict__ owner8,
+                                                const unsigned char *__restrict__ owner,
                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
                                                 float *__restrict__ P, int M, int ts, int64_t r0, int rpw, int lane) {
     using U = typename L::U;
@@ -293,7 +293,7 @@ __device__ __forceinline__ void short_rows_body(const void *__restrict__ A, cons
         len = rowptr[r0 + lane + 1] - rs;
         if (len >= ts) len = 0;
         // rows computed by the dense-tile or the row-panel path
-        if (owner8 && owner8[(r0 + lane) >> 3] != 0) len = 0;
+        if (owner && owner[r0 + lane] != 0) len = 0;
     }
     int incl = len;
     for (int o = 1; o < WAVE; o <<= 1) {
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(BLOCK) void k_short_rows(const void *__restrict__ A
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                 const int32_t *__restrict__ rowptr,
-                                                const unsigned char *__restrict__ owner8,
+                                                const unsigned char *__restrict__ owner,
                                                 const int32_t *__restrict__ col,
                                                 const float *__restrict__ sval, float *__restrict__ P, int M,
                                                 int ts, int rpw, int64_t short_blocks,
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, cons
         const int64_t sb = blk - items_before;
         const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
         if (r0 >= M) return;
-        short_rows_body<L>(A, B, KU, rowptr, owner8, col, sval, P, M, ts, r0, rpw, lane_id());
+        short_rows_body<L>(A, B, KU, rowptr, owner, col, sval, P, M, ts, r0, rpw, lane_id());
     }
 }
 

@@ -32,7 +32,8 @@ enum CounterKind {
 };
 struct DevCounters {
     unsigned int bad_pattern, coo_unsorted, pad0, pad1;
-    unsigned long long n_items, tiles_scanned, panel_items, pad2;   // scan totals, one writer each
+    unsigned long long n_items, tiles_scanned, panel_items;          // scan totals, one writer each
+    unsigned long long n_candidates;                                 // rows offered to the gathered strips
     unsigned int max_len[SPREAD];
     unsigned long long k[K_KINDS][SPREAD];
 };
@@ -176,12 +177,13 @@ constexpr int SCAN_BLOCK = 256;
 constexpr int SCAN_ITEMS = 4;                       // rows per thread
 constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;  // rows per block
 
-// owner8 (may be null): one byte per group of 8 rows, non-zero when the dense-tile
-// path (1) or the row-panel path (2) computes those rows; they count as empty here
+// owner (may be null): one byte per row, non-zero when the dense-tile path (1: a
+// 16-row strip, 3: a strip of rows gathered by column window) or the row-panel path
+// (2) computes the row; such rows count as empty here
 __device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr,
-                                                       const unsigned char *__restrict__ owner8, int64_t i,
+                                                       const unsigned char *__restrict__ owner, int64_t i,
                                                        int M, int ts, int seg, unsigned int *len_out) {
-    if (i >= M || (owner8 && owner8[i >> 3] != 0)) { *len_out = 0; return 0; }
+    if (i >= M || (owner && owner[i] != 0)) { *len_out = 0; return 0; }
     const unsigned int len = (unsigned int)(rowptr[i + 1] - rowptr[i]);
     *len_out = len;
     return len >= (unsigned int)ts ? (len + seg - 1) / seg : 0u;
@@ -212,7 +214,7 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 
 // pass 1: items per block of SCAN_TILE rows, plus the row statistics
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
-                                                               const unsigned char *__restrict__ owner8, int M,
+                                                               const unsigned char *__restrict__ owner, int M,
                                                                int ts, int seg, unsigned int *__restrict__ block_sums,
                                                                DevCounters *pc) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
@@ -220,7 +222,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        const unsigned int cnt = row_item_count(rowptr, owner8, base + q, M, ts, seg, &len);
+        const unsigned int cnt = row_item_count(rowptr, owner, base + q, M, ts, seg, &len);
         items += cnt;
         if (len == 0) continue;
         if (cnt == 0) { ++r_short; n_short += len; }
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__
 
 // pass 3: write the items
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr,
-                                                               const unsigned char *__restrict__ owner8, int M,
+                                                               const unsigned char *__restrict__ owner, int M,
                                                                int ts, int seg,
                                                                const unsigned int *__restrict__ block_offsets,
                                                                RowItem *__restrict__ items) {
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
     unsigned int cnt[SCAN_ITEMS], mine = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        cnt[q] = row_item_count(rowptr, owner8, base + q, M, ts, seg, &len);
+        cnt[q] = row_item_count(rowptr, owner, base + q, M, ts, seg, &len);
         mine += cnt[q];
     }
     unsigned int total;
@@ -294,16 +296,16 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
 // Row-panel detector: panel p = rows [8p, 8p+8).  It qualifies when all 8 rows
 // exist, are not owned by the dense-tile path, have the same length >= min_len and
 // the same column list.  One wavefront per panel; lanes stride over the list.
-// counts[p] = work items of the panel (ceil(len/pseg)) or 0; owner8[p] = 2 when taken.
+// counts[p] = work items of the panel (ceil(len/pseg)) or 0; owner = 2 on its rows when taken.
 __global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__ rowptr,
                                                      const int32_t *__restrict__ col, int M, int64_t n_panels,
-                                                     int min_len, int pseg, unsigned char *__restrict__ owner8,
+                                                     int min_len, int pseg, unsigned char *__restrict__ owner,
                                                      unsigned int *__restrict__ counts, DevCounters *pc) {
     const int64_t p = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     if (p >= n_panels) return;
     const int lane = lane_id();
     const int64_t row0 = p * 8;
-    bool ok = row0 + 8 <= M && owner8[p] == 0;
+    bool ok = row0 + 8 <= M && owner[row0] == 0;   // strips own aligned groups of 16 rows
     int s0 = 0, len = 0;
     if (ok) {
         s0 = rowptr[row0];
@@ -326,10 +328,10 @@ __global__ __launch_bounds__(256) void k_panel_flags(const int32_t *__restrict__
         }
         ok = __ballot(differ) == 0;
     }
+    if (ok && lane < 8) owner[row0 + lane] = 2;
     if (lane == 0) {
         counts[p] = ok ? (unsigned int)((len + pseg - 1) / pseg) : 0u;
         if (ok) {
-            owner8[p] = 2;
             spread_add(pc, K_PANELS, 1ull);
             spread_add(pc, K_NNZ_PANELS, (unsigned long long)len * 8ull);
         }

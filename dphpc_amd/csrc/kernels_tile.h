@@ -21,6 +21,7 @@
 // entries, and far fewer at the 25-100 % fill it is used for.
 #pragma once
 #include "device_utils.h"
+#include "kernels_gather.h"
 #include "kernels_plan.h"
 
 namespace sddmm {
@@ -226,7 +227,7 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
 // (sorted rows, at least min_fill entries per tile on average), else 0.
 __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips, int min_fill,
-    unsigned int *__restrict__ strip_ntiles, unsigned char *__restrict__ owner8, DevCounters *pc) {
+    unsigned int *__restrict__ strip_ntiles, unsigned char *__restrict__ owner, DevCounters *pc) {
     __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
     const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
     if (strip >= n_strips) return;            // whole waves leave
@@ -276,11 +277,10 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
         }
         take = tiles > 0 && tiles <= max_tiles && entries >= (int64_t)min_fill * tiles;
     }
+    if (take && lane < 16 && strip * 16 + lane < M) owner[strip * 16 + lane] = 1;
     if (lane == 0) {
         strip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
         if (take) {
-            owner8[2 * strip] = 1;         // both 8-row halves (the array is padded to an even length)
-            owner8[2 * strip + 1] = 1;
             spread_add(pc, K_TILES, (unsigned long long)tiles);
             spread_add(pc, K_NNZ_TILES, (unsigned long long)entries);
         }
@@ -348,10 +348,167 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
     }
 }
 
+// ---- gathered strips ---------------------------------------------------------------
+// Rows that are dense inside a column window need not be neighbours to share tiles:
+// any 16 rows whose windows overlap form a strip for the matrix cores as well as 16
+// consecutive ones do.  Candidate rows (not owned yet, at least min_len entries that
+// fill a quarter of their column span or more) are sorted by their first column;
+// every 16 consecutive rows of that order are one gathered strip, classified with
+// the same bitmap and threshold as a natural strip.  TileDesc.strip of such a strip
+// is GATHERED_BASE + its index, its rows are listed in a table (16 per strip, -1 for
+// a missing row).
+constexpr int GATHERED_BASE = 1 << 30;
+
+__global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__restrict__ rowptr,
+                                                           const int32_t *__restrict__ col, int M,
+                                                           const unsigned char *__restrict__ owner, int min_len,
+                                                           unsigned int *__restrict__ keys, int32_t *__restrict__ rows,
+                                                           unsigned long long *__restrict__ count) {
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bool cand = false;
+    int first = 0;
+    if (r < M && owner[r] == 0) {
+        const int s = rowptr[r], e = rowptr[r + 1];
+        if (e - s >= min_len) {
+            first = col[s];
+            const int64_t span = (int64_t)col[e - 1] - first + 1;
+            cand = span > 0 && (int64_t)(e - s) * 4 >= span;
+        }
+    }
+    // one append per wave
+    const unsigned long long m = __ballot(cand);
+    if (m == 0ull) return;
+    const int lane = lane_id();
+    unsigned long long base = 0;
+    if (lane == 0) base = atomicAdd(count, (unsigned long long)__popcll(m));
+    base = ((unsigned long long)(unsigned int)__builtin_amdgcn_readfirstlane((int)(base >> 32)) << 32) |
+           (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+    if (cand) {
+        const unsigned long long at = base + (unsigned long long)__popcll(m & ((1ull << lane) - 1ull));
+        keys[at] = (unsigned int)first;
+        rows[at] = (int32_t)r;
+    }
+}
+
+// Rows, extent and column span of gathered strip vs; lanes 0..15 keep one row each.
+struct GatheredHead {
+    int row, s, e;        // per lane (row -1: none)
+    int lo, span;         // wave-uniform, in tile columns
+    int64_t entries;      // wave-uniform
+};
+__device__ __forceinline__ GatheredHead gathered_head(const int32_t *__restrict__ rowptr,
+                                                      const int32_t *__restrict__ col,
+                                                      const int32_t *__restrict__ sorted_rows, int64_t n_cand,
+                                                      int64_t vs) {
+    GatheredHead h;
+    const int lane = lane_id();
+    const int64_t idx = vs * 16 + lane;
+    h.row = lane < 16 && idx < n_cand ? sorted_rows[idx] : -1;
+    h.s = h.row >= 0 ? rowptr[h.row] : 0;
+    h.e = h.row >= 0 ? rowptr[h.row + 1] : 0;
+    const bool has = h.e > h.s;
+    const int first = has ? (col[h.s] >> 4) : INT32_MAX;
+    const int last = has ? (col[h.e - 1] >> 4) : -1;
+    // lanes 16..63 hold the neutral values, so the 16-lane reductions of row 0 are the strip's
+    const int l = __builtin_amdgcn_readfirstlane(min16(first));
+    const int hneg = __builtin_amdgcn_readfirstlane(min16(-last));
+    h.lo = l;
+    h.span = l == INT32_MAX ? 0 : -hneg - l + 1;
+    h.entries = (int64_t)__builtin_amdgcn_readfirstlane(sum16(h.e - h.s));
+    return h;
+}
+
+// marks the tile columns of the strip's 16 rows in bm; false when a row is not sorted
+__device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, const GatheredHead &h, unsigned int *bm) {
+    const int lane = lane_id();
+    const int words = (h.span + 31) >> 5;
+    for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
+    wave_lds_order();
+    bool sorted = true;
+    for (int i = 0; i < 16; ++i) {
+        const int si = __builtin_amdgcn_readlane(h.s, i), ei = __builtin_amdgcn_readlane(h.e, i);
+        if (ei <= si) continue;                  // wave-uniform
+        int64_t descents = 0;
+        (void)strip_scan<true>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
+        sorted = sorted && descents == 0;
+    }
+    wave_lds_order();
+    return sorted;
+}
+
+// pass 1 of the gathered strips: tiles per strip (0: not taken), the strip's row
+// table, ownership of the rows of a taken strip.
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_count(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, const int32_t *__restrict__ sorted_rows,
+    int64_t n_cand, int64_t n_vstrips, int min_fill, unsigned int *__restrict__ vstrip_ntiles,
+    int32_t *__restrict__ vrows, unsigned char *__restrict__ owner, DevCounters *pc) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
+    const int64_t vs = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
+    if (vs >= n_vstrips) return;
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const GatheredHead h = gathered_head(rowptr, col, sorted_rows, n_cand, vs);
+    if (lane < 16) vrows[vs * 16 + lane] = h.row;
+    int64_t tiles = 0;
+    bool take = false;
+    if (h.span > 0 && h.span <= STRIP_BM_WORDS * 32 && h.entries >= min_fill) {
+        const bool sorted = gathered_mark(col, h, bm);
+        const int words = (h.span + 31) >> 5;
+        int t = 0;
+        for (int w = lane; w < words; w += WAVE) t += __builtin_popcount(bm[w]);
+        tiles = wave_sum_i32(t);
+        take = sorted && tiles > 0 && h.entries >= (int64_t)min_fill * tiles;
+    }
+    if (take && h.row >= 0) owner[h.row] = 3;
+    if (lane == 0) {
+        vstrip_ntiles[vs] = take ? (unsigned int)tiles : 0u;
+        if (take) {
+            spread_add(pc, K_TILES, (unsigned long long)tiles);
+            spread_add(pc, K_NNZ_TILES, (unsigned long long)h.entries);
+        }
+    }
+}
+
+// pass 2 of the gathered strips: strip and tile column of every descriptor
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_tiles(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, const int32_t *__restrict__ sorted_rows,
+    int64_t n_cand, int64_t n_vstrips, const unsigned int *__restrict__ vstrip_ntiles,
+    const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
+    const int64_t vs = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
+    if (vs >= n_vstrips) return;
+    if (vstrip_ntiles[vs] == 0) return;
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const GatheredHead h = gathered_head(rowptr, col, sorted_rows, n_cand, vs);
+    (void)gathered_mark(col, h, bm);
+    const int words = (h.span + 31) >> 5;
+    int64_t run = vstrip_off[vs];
+    for (int wb = 0; wb < words; wb += WAVE) {
+        const int w = wb + lane;
+        unsigned int x = w < words ? bm[w] : 0u;
+        const int n = __builtin_popcount(x);
+        int incl = n;
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const int up = __shfl_up(incl, o, WAVE);
+            if (lane >= o) incl += up;
+        }
+        int64_t at = run + (incl - n);
+        while (x) {
+            const int b = __builtin_ctz(x);
+            x &= x - 1;
+            *reinterpret_cast<int4 *>(tiles + at) = make_int4(GATHERED_BASE + (int)vs, h.lo + w * 32 + b, 0, 0);
+            ++at;
+        }
+        run += __builtin_amdgcn_readlane(incl, WAVE - 1);
+    }
+}
+
 // pass 3: one thread per (descriptor, row): CSR position of the row's first entry
 // at or after the tile's first column, and the mask of the tile's columns present.
 __global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ rowptr,
                                                    const int32_t *__restrict__ col, int M,
+                                                   const int32_t *__restrict__ vrows,
                                                    TileDesc *__restrict__ tiles, int64_t n_tiles) {
     const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t t = slot >> 4;
@@ -361,9 +518,10 @@ __global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ r
     const int4 head = *reinterpret_cast<const int4 *>(d);     // strip, tj, pad[0], pad[1]
     if (head.z != 0) return;                                   // written by the merging walk
     const int tj = head.y;
-    const int64_t row = (int64_t)head.x * 16 + sub;
+    const int64_t row = head.x >= GATHERED_BASE ? (int64_t)vrows[(int64_t)(head.x - GATHERED_BASE) * 16 + sub]
+                                                : (int64_t)head.x * 16 + sub;
     int p = 0, end = 0;
-    if (row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
+    if (row >= 0 && row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
     const int target = tj * 16;
     int a = p, b = end;
     while (a < b) {
@@ -432,14 +590,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //   and then computes    MFMAs of tile t, scale, scatter (operands landed during t-1)
 // The A panel of the current strip stays in registers and is reloaded only when
 // the strip changes (a wave-uniform branch placed before the iteration's loads).
+// tiles [w*tiles_per_wave, (w+1)*tiles_per_wave) on the calling wavefront
 template <int DT, int STEPS>
-__global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
-                                                const TileDesc *__restrict__ tiles, int64_t n_tiles,
-                                                int tiles_per_wave, const float *__restrict__ sval,
-                                                float *__restrict__ P, int64_t nblocks) {
-    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
-    if (blk < 0) return;
-    const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
+__device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                          const int32_t *__restrict__ vrows, const TileDesc *__restrict__ tiles,
+                                          int64_t n_tiles, int tiles_per_wave, const float *__restrict__ sval,
+                                          float *__restrict__ P, int64_t w) {
     int64_t t = w * tiles_per_wave;
     if (t >= n_tiles) return;
     int64_t t_end = t + tiles_per_wave;
@@ -513,8 +669,9 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
         const int strip = __builtin_amdgcn_readfirstlane(d_cur.strip);
         if (strip != cur_strip) {
             cur_strip = strip;
-            int64_t arow = (int64_t)strip * 16 + lrow;
-            arow = arow < M ? arow : M - 1;   // rows past M are never in a mask
+            int64_t arow = strip >= GATHERED_BASE ? (int64_t)vrows[(int64_t)(strip - GATHERED_BASE) * 16 + lrow]
+                                                  : (int64_t)strip * 16 + lrow;
+            arow = arow < 0 ? 0 : (arow < M ? arow : M - 1);   // missing rows are never in a mask
             const uint4 *src = Au + arow * ROW_UNITS + lunit;
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) a[s] = to_operand(src[s * 4]);
@@ -549,6 +706,61 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
         o_cur = o_nxt;
         d_cur = d_nxt;
         d_nxt = d_nn;
+    }
+}
+
+template <int DT, int STEPS>
+__global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                                const int32_t *__restrict__ vrows,
+                                                const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                int tiles_per_wave, const float *__restrict__ sval,
+                                                float *__restrict__ P, int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    tile_wave<DT, STEPS>(A, B, M, N, vrows, tiles, n_tiles, tiles_per_wave, sval, P,
+                         blk * WAVES_PER_BLOCK + wave_in_block());
+}
+
+// AUTO in one launch when a matrix has tiles and rows: logical blocks are dealt out
+// evenly between tile blocks (tile_wave), segment-item blocks and short-row blocks,
+// so that every XCD gets its share of each.  Kernels of one stream run one after
+// the other; two short launches leave the chip half idle twice, one launch does not.
+// L must be the full-K, 32-bit-offset layout of a row of STEPS * 64 bytes.
+template <class L, int STEPS>
+__global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                      const int32_t *__restrict__ rowptr,
+                                                      const unsigned char *__restrict__ owner,
+                                                      const int32_t *__restrict__ col,
+                                                      const float *__restrict__ sval, float *__restrict__ P, int M,
+                                                      int N, int ts, int rpw, int64_t short_blocks,
+                                                      const RowItem *__restrict__ items, int64_t n_items,
+                                                      const int32_t *__restrict__ vrows,
+                                                      const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                      int tiles_per_wave, int64_t tile_blocks, int64_t nblocks) {
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t tiles_before = blk * tile_blocks / nblocks;
+    if (((blk + 1) * tile_blocks / nblocks) != tiles_before) {
+        tile_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tiles, n_tiles, tiles_per_wave, sval, P,
+                                   tiles_before * WAVES_PER_BLOCK + wave_in_block());
+        return;
+    }
+    const int64_t rb = blk - tiles_before, rest = nblocks - tile_blocks;
+    const int64_t item_blocks = rest - short_blocks;
+    const int64_t items_before = rb * item_blocks / rest;
+    if (((rb + 1) * item_blocks / rest) != items_before) {
+        const int64_t w = items_before * WAVES_PER_BLOCK + wave_in_block();
+        if (w >= n_items) return;
+        const RowItem it = items[w];
+        const int row = __builtin_amdgcn_readfirstlane(it.row);
+        const int start = __builtin_amdgcn_readfirstlane(it.start);
+        const int end = __builtin_amdgcn_readfirstlane(it.end);
+        row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
+    } else {
+        const int64_t sb = rb - items_before;
+        const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
+        if (r0 >= M) return;
+        short_rows_body<L>(A, B, KU, rowptr, owner, col, sval, P, M, ts, r0, rpw, lane_id());
     }
 }
 

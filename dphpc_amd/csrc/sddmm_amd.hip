@@ -4,6 +4,10 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
@@ -24,6 +28,7 @@ struct sddmm_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+
     char err[512] = {0};
 
     // dense operands
@@ -64,8 +69,16 @@ struct sddmm_ctx {
     int64_t n_tiles = 0, tiles_cap = 0, nnz_tiles = 0;
     int tile_steps = 0, tiles_per_wave = 8;
     bool tiles_active = false;       // d_tiles describes the current pattern
-    // row ownership (one byte per 8 rows: 0 rows kernels, 1 dense tiles, 2 row panels)
-    unsigned char *d_owner8 = nullptr;
+    int64_t n_tiles_natural = 0;     // descriptors of 16-row strips come first, gathered strips after
+    // gathered strips: candidate rows, sorted by first column, 16 per strip
+    unsigned int *d_cand_keys = nullptr, *d_sorted_keys = nullptr;
+    int32_t *d_cand_rows = nullptr, *d_sorted_rows = nullptr, *d_vrows = nullptr;
+    void *d_sort_tmp = nullptr;
+    size_t sort_tmp_bytes = 0;
+    int64_t cand_cap = 0, vstrips_cap = 0, n_cand = 0, n_vstrips = 0;
+    unsigned int *d_vstrip_ntiles = nullptr, *d_vstrip_off = nullptr;
+    // row ownership (one byte per row: 0 row kernels, 1 dense tiles, 2 row panels, 3 gathered strips)
+    unsigned char *d_owner = nullptr;
     int64_t owner_cap = 0;
     bool owner_active = false;
     // row-panel path
@@ -130,7 +143,11 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_strip_ntiles);
     dfree(c->d_strip_off);
     dfree(c->d_tiles);
-    dfree(c->d_owner8);
+    dfree(c->d_cand_keys); dfree(c->d_sorted_keys); dfree(c->d_cand_rows); dfree(c->d_sorted_rows);
+    dfree(c->d_vrows); dfree(c->d_sort_tmp); dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off);
+    c->sort_tmp_bytes = 0;
+    c->cand_cap = c->vstrips_cap = c->n_cand = c->n_vstrips = 0;
+    dfree(c->d_owner);
     dfree(c->d_panel_counts);
     dfree(c->d_panel_off);
     dfree(c->d_panel_items);
@@ -284,6 +301,36 @@ void launch_short_rows(sddmm_ctx *c, int ts, int rpw) {
     });
 }
 
+// Tiles and rows in one launch (k_auto_tiles): rows of 64 to 256 bytes, where both
+// kernels are short and their register needs are alike.  Returns false when the
+// layout has no fused kernel; the caller then launches the two kernels in turn.
+bool launch_auto_with_tiles(sddmm_ctx *c) {
+    const Shape s = shape_of(c);
+    if (c->tile_steps < 1 || c->tile_steps > 4 || !s.fullk || s.wide || s.unit == 1 || s.KU != 4 * c->tile_steps)
+        return false;
+    const int64_t waves = c->rows_short > 0 ? ((int64_t)c->sM + c->rpw - 1) / c->rpw : 0;
+    const int64_t short_blocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t tile_waves = (c->n_tiles + c->tiles_per_wave - 1) / c->tiles_per_wave;
+    const int64_t tile_blocks = (tile_waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t nblocks = short_blocks + item_blocks + tile_blocks;
+    bool launched = false;
+    with_layout(s, [&](auto L) {
+        using LT = decltype(L);
+        constexpr int KU_ = LT::LPN * LT::UPL;
+        if constexpr (!LT::LONG && LT::FULLK && !LT::WIDE && LT::U::ELEMS > 1 && (KU_ == 4 || KU_ == 8 || KU_ == 16)) {
+            hipLaunchKernelGGL((k_auto_tiles<LT, KU_ / 4>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                               (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
+                               (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
+                               c->dP, c->sM, c->N, c->ts, c->rpw, short_blocks, c->d_items, c->n_items,
+                               (const int32_t *)c->d_vrows, (const TileDesc *)c->d_tiles, c->n_tiles,
+                               c->tiles_per_wave, tile_blocks, nblocks);
+            launched = true;
+        }
+    });
+    return launched;
+}
+
 void launch_auto(sddmm_ctx *c) {
     const Shape s = shape_of(c);
     const int64_t waves = c->rows_short > 0 ? ((int64_t)c->sM + c->rpw - 1) / c->rpw : 0;
@@ -294,7 +341,7 @@ void launch_auto(sddmm_ctx *c) {
         using LT = decltype(L);
         hipLaunchKernelGGL((k_auto<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
-                           (const unsigned char *)(c->owner_active ? c->d_owner8 : nullptr), c->d_col, c->d_sval,
+                           (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
                            c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
     });
 }
@@ -317,7 +364,7 @@ int classify_rows(sddmm_ctx *c) {
                               sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     if (nb > 0) {
-        const unsigned char *owner = c->owner_active ? c->d_owner8 : nullptr;
+        const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
         hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, owner,
                            c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc);
         hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
@@ -337,7 +384,7 @@ int classify_rows(sddmm_ctx *c) {
     }
     if (c->n_items > 0) {
         hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
-                           (const unsigned char *)(c->owner_active ? c->d_owner8 : nullptr), c->sM, c->ts, c->seg,
+                           (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts, c->seg,
                            c->d_block_sums, c->d_items);
         HIP_TRY(c, hipGetLastError());
     }
@@ -362,33 +409,42 @@ int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t
 
 // Clears the row-ownership bytes and the tile / panel counters before the classifiers run.
 int begin_ownership(sddmm_ctx *c) {
-    const int64_t bytes = 2 * (((int64_t)c->sM + 15) / 16) + 16;
+    const int64_t bytes = (int64_t)c->sM + 64;
     if (bytes > c->owner_cap) {
-        dfree(c->d_owner8);
-        ALLOC_TRY(c, c->d_owner8, (size_t)bytes);
+        dfree(c->d_owner);
+        ALLOC_TRY(c, c->d_owner, (size_t)bytes);
         c->owner_cap = bytes;
     }
-    HIP_TRY(c, hipMemsetAsync(c->d_owner8, 0, (size_t)bytes, c->stream));
+    HIP_TRY(c, hipMemsetAsync(c->d_owner, 0, (size_t)bytes, c->stream));
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_TILES][0], 0,
                               sizeof(unsigned long long) * SPREAD * (K_NNZ_PANELS - K_TILES + 1), c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 2 * sizeof(unsigned long long), c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 3 * sizeof(unsigned long long), c->stream));
     c->owner_active = true;
     c->tiles_active = false;
-    c->n_tiles = c->nnz_tiles = 0;
+    c->n_tiles = c->nnz_tiles = c->n_tiles_natural = 0;
+    c->n_cand = c->n_vstrips = 0;
     c->n_panel_items = c->n_panels = c->nnz_panels = 0;
     return SDDMM_OK;
 }
 
-// Dense-tile classifier.  min_fill = average stored entries per 16x16 tile a strip
-// needs to be taken.  Leaves tiles_active false when the path does not apply
-// (row size not a multiple of 64 bytes, nothing qualifies).
-int plan_tiles(sddmm_ctx *c, int min_fill) {
-    if (c->nnz == 0) return SDDMM_OK;
+// Dense-tile classifier, in three steps so that the row panels can be looked for in
+// between: (1) 16-row strips, (2) strips of rows gathered by column window among the
+// rows nobody owns yet, (3) descriptors of both.  min_fill = average stored entries
+// per 16x16 tile a strip needs to be taken.  tile_steps stays 0 when the path does not
+// apply (row size not a multiple of 64 bytes).
+bool tile_path_applies(sddmm_ctx *c) {
+    c->tile_steps = 0;
+    if (c->nnz == 0) return false;
     const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
-    if (row_bytes % 64) return SDDMM_OK;
+    if (row_bytes % 64) return false;
     const int steps = (int)(row_bytes / 64);
-    if (steps != 1 && steps != 2 && steps != 4 && steps != 8 && steps != 16) return SDDMM_OK;
+    if (steps != 1 && steps != 2 && steps != 4 && steps != 8 && steps != 16) return false;
     c->tile_steps = steps;
+    return true;
+}
+
+int plan_tiles_count(sddmm_ctx *c, int min_fill) {
+    if (!tile_path_applies(c)) return SDDMM_OK;
     const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
     if (n_strips > c->strips_cap) {
         dfree(c->d_strip_ntiles);
@@ -399,27 +455,98 @@ int plan_tiles(sddmm_ctx *c, int min_fill) {
     }
     const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
     hipLaunchKernelGGL(k_strip_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
-                       c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner8, c->d_pc);
+                       c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner, c->d_pc);
     HIP_TRY(c, hipGetLastError());
     int rc = device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
     if (rc) return rc;
     rc = fetch_counters(c);
     if (rc) return rc;
-    c->n_tiles = (int64_t)c->pc.n_tiles;
+    c->n_tiles = c->n_tiles_natural = (int64_t)c->pc.n_tiles;
     c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
     if ((int64_t)c->pc.tiles_scanned != c->n_tiles)
         return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
+    return SDDMM_OK;
+}
+
+int plan_gathered_count(sddmm_ctx *c, int min_fill, int min_len) {
+    if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
+    const int64_t M = c->sM;
+    if (M > c->cand_cap) {
+        dfree(c->d_cand_keys); dfree(c->d_sorted_keys); dfree(c->d_cand_rows); dfree(c->d_sorted_rows);
+        ALLOC_TRY(c, c->d_cand_keys, (size_t)M * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_sorted_keys, (size_t)M * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_cand_rows, (size_t)M * sizeof(int32_t));
+        ALLOC_TRY(c, c->d_sorted_rows, (size_t)M * sizeof(int32_t));
+        c->cand_cap = M;
+    }
+    hipLaunchKernelGGL(k_gather_candidates, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, c->stream, c->d_rowptr,
+                       c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys, c->d_cand_rows,
+                       &c->d_pc->n_candidates);
+    HIP_TRY(c, hipGetLastError());
+    int rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_cand = (int64_t)c->raw.n_candidates;
+    if (c->n_cand < 2) { c->n_cand = 0; return SDDMM_OK; }
+    // candidates ordered by first column (the append order of the candidates is not
+    // deterministic, the sorted order of equal keys therefore is not either: only the
+    // grouping into strips can differ between plans, never a result)
+    size_t need = 0;
+    HIP_TRY(c, rocprim::radix_sort_pairs(nullptr, need, c->d_cand_keys, c->d_sorted_keys, c->d_cand_rows,
+                                         c->d_sorted_rows, (size_t)c->n_cand, 0, 32, c->stream));
+    if (need > c->sort_tmp_bytes) {
+        dfree(c->d_sort_tmp);
+        ALLOC_TRY(c, c->d_sort_tmp, need);
+        c->sort_tmp_bytes = need;
+    }
+    HIP_TRY(c, rocprim::radix_sort_pairs(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, c->d_cand_rows,
+                                         c->d_sorted_rows, (size_t)c->n_cand, 0, 32, c->stream));
+    c->n_vstrips = (c->n_cand + 15) / 16;
+    if (c->n_vstrips > c->vstrips_cap) {
+        dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off); dfree(c->d_vrows);
+        ALLOC_TRY(c, c->d_vstrip_ntiles, (size_t)c->n_vstrips * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_vstrip_off, (size_t)c->n_vstrips * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_vrows, (size_t)c->n_vstrips * 16 * sizeof(int32_t));
+        c->vstrips_cap = c->n_vstrips;
+    }
+    const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+    hipLaunchKernelGGL(k_gathered_count, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr, c->d_col,
+                       (const int32_t *)c->d_sorted_rows, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
+                       c->d_vrows, c->d_owner, c->d_pc);
+    HIP_TRY(c, hipGetLastError());
+    rc = device_scan(c, c->d_vstrip_ntiles, c->d_vstrip_off, c->n_vstrips, &c->d_pc->tiles_scanned);
+    if (rc) return rc;
+    rc = fetch_counters(c);
+    if (rc) return rc;
+    c->n_tiles = (int64_t)c->pc.n_tiles;
+    c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
+    if ((int64_t)c->pc.tiles_scanned != c->n_tiles - c->n_tiles_natural)
+        return fail(c, SDDMM_ERR_HIP, "internal: gathered tile scan disagrees with tile count");
+    return SDDMM_OK;
+}
+
+int plan_tiles_fill(sddmm_ctx *c) {
     if (c->n_tiles == 0) return SDDMM_OK;
     if (c->n_tiles > c->tiles_cap) {
         dfree(c->d_tiles);
         ALLOC_TRY(c, c->d_tiles, (size_t)c->n_tiles * sizeof(TileDesc));
         c->tiles_cap = c->n_tiles;
     }
-    hipLaunchKernelGGL(k_strip_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
-                       c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
-    HIP_TRY(c, hipGetLastError());
+    if (c->n_tiles_natural > 0) {
+        const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
+        const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+        hipLaunchKernelGGL(k_strip_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                           c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
+        HIP_TRY(c, hipGetLastError());
+    }
+    if (c->n_tiles > c->n_tiles_natural) {
+        const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+        hipLaunchKernelGGL(k_gathered_tiles, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                           c->d_col, (const int32_t *)c->d_sorted_rows, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
+                           c->d_vstrip_off, c->d_tiles + c->n_tiles_natural);
+        HIP_TRY(c, hipGetLastError());
+    }
     hipLaunchKernelGGL(k_tile_rows, dim3((unsigned)((c->n_tiles * 16 + 255) / 256)), dim3(256), 0, c->stream,
-                       c->d_rowptr, c->d_col, c->sM, c->d_tiles, c->n_tiles);
+                       c->d_rowptr, c->d_col, c->sM, (const int32_t *)c->d_vrows, c->d_tiles, c->n_tiles);
     HIP_TRY(c, hipGetLastError());
     c->tiles_active = true;
     c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 4));
@@ -458,7 +585,7 @@ int plan_panels(sddmm_ctx *c, int min_len, int pseg) {
         c->panels_cap = n_panels;
     }
     hipLaunchKernelGGL(k_panel_flags, dim3((unsigned)((n_panels * WAVE + 255) / 256)), dim3(256), 0, c->stream,
-                       c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner8, c->d_panel_counts, c->d_pc);
+                       c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner, c->d_panel_counts, c->d_pc);
     HIP_TRY(c, hipGetLastError());
     int rc = device_scan(c, c->d_panel_counts, c->d_panel_off, n_panels, &c->d_pc->panel_items);
     if (rc) return rc;
@@ -529,7 +656,8 @@ void launch_tile_t(sddmm_ctx *c) {
     const int64_t waves = (c->n_tiles + c->tiles_per_wave - 1) / c->tiles_per_wave;
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     hipLaunchKernelGGL((k_tile<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
-                       (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const TileDesc *)c->d_tiles, c->n_tiles,
+                       (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
+                       (const TileDesc *)c->d_tiles, c->n_tiles,
                        c->tiles_per_wave, (const float *)c->d_sval, c->dP, nblocks);
 }
 template <int DT>
@@ -595,12 +723,20 @@ int enqueue_run(sddmm_ctx *c) {
     switch (c->strategy) {
         case SDDMM_AUTO:
         case SDDMM_MFMA_TILE:
-        case SDDMM_LDS_TILED:
+        case SDDMM_LDS_TILED: {
+            // (a second stream for the first of these independent kernels was measured:
+            // the fork/join events cost more than the overlap returns, 33 us against 23 us
+            // on the mixed-density shape)
             c->launches = 0;
-            if (c->tiles_active && c->n_tiles > 0) { launch_tiles(c); ++c->launches; }
+            const bool tiles = c->tiles_active && c->n_tiles > 0, rows = c->rows_short > 0 || c->n_items > 0;
+            bool fused = false;
+            if (tiles && rows && env_int("SDDMM_FUSE", 1) != 0) fused = launch_auto_with_tiles(c);
+            if (fused) ++c->launches;
+            if (tiles && !fused) { launch_tiles(c); ++c->launches; }
             if (c->n_panel_items > 0) { launch_panels(c); ++c->launches; }
-            if (c->rows_short > 0 || c->n_items > 0) { launch_auto(c); ++c->launches; }
+            if (rows && !fused) { launch_auto(c); ++c->launches; }
             break;
+        }
         case SDDMM_FLAT: launch_flat(c); break;
         case SDDMM_ROW_WAVE: launch_row_wave(c, nullptr, c->sM); break;
         case SDDMM_SHORT_ROWS:
@@ -640,13 +776,30 @@ int do_plan(sddmm_ctx *c, int strategy) {
             if (!csr_ok) return fail(c, SDDMM_ERR_UNSUPPORTED, "strategy %d needs row-sorted entries", resolved);
             int rc = begin_ownership(c);
             if (rc) return rc;
+            // entries per 16x16 tile from which the tile kernel beats the gather kernels,
+            // measured on banded matrices of varying fill: 74 at 128-byte rows, 50 at 256
+            // and 512 bytes; 64-byte rows keep the older, conservative figure
+            const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
+            const int tile_fill = std::max(1, env_int("SDDMM_TILE_FILL", row_bytes <= 64 ? 96 : row_bytes <= 128 ? 80 : 56));
             if (resolved != SDDMM_LDS_TILED) {
-                rc = plan_tiles(c, resolved == SDDMM_MFMA_TILE ? 1 : std::max(1, env_int("SDDMM_TILE_FILL", 96)));
+                // 16-row strips are looked at before the row panels and must not take what the
+                // panel kernel does better (8x8-block rows reach ~80 entries per tile); the
+                // strips gathered after the panels use the measured break-even
+                rc = plan_tiles_count(c, resolved == SDDMM_MFMA_TILE ? 1 : std::max(96, tile_fill));
                 if (rc) return rc;
             }
             if (resolved != SDDMM_MFMA_TILE) {
                 rc = plan_panels(c, resolved == SDDMM_LDS_TILED ? 1 : std::max(1, env_int("SDDMM_PANEL_MIN", 16)),
                                  std::max(WAVE, env_int("SDDMM_PANEL_SEG", 512)));
+                if (rc) return rc;
+            }
+            if (resolved == SDDMM_AUTO && env_int("SDDMM_GATHERED", 1) != 0) {
+                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)),
+                                         std::max(16, env_int("SDDMM_GATHERED_MIN", 64)));
+                if (rc) return rc;
+            }
+            if (resolved != SDDMM_LDS_TILED) {
+                rc = plan_tiles_fill(c);
                 if (rc) return rc;
             }
             c->ts = std::max(1, env_int("SDDMM_TS", 24));

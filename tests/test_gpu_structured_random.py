@@ -119,10 +119,12 @@ def _host_tile_model(M, rowptr, col, min_fill):
 
 
 @pytest.mark.parametrize("seed", range(12))
-def test_strip_classifier_matches_host_model(engine_factory, seed):
+def test_strip_classifier_matches_host_model(engine_factory, monkeypatch, seed):
     """Tile counts and covered entries reported by the device classifier against the
     host model, on matrices whose strips mix clustered, scattered, unsorted and
-    duplicated rows (K=16: 64-byte rows, so the tile path applies)."""
+    duplicated rows (K=16: 64-byte rows, so the tile path applies).  Strips of
+    gathered rows are switched off for the comparison and checked on top of it."""
+    monkeypatch.setenv("SDDMM_GATHERED", "0")
     rng = np.random.default_rng(7000 + seed)
     N = int(rng.choice([100, 1000, 40000, 600_000]))
     M = int(rng.integers(17, 400))
@@ -177,4 +179,16 @@ def test_strip_classifier_matches_host_model(engine_factory, seed):
             assert want_tiles == 0
         ok, worst, i = O.check_values(e.values(), ref, mag=mag)
         assert ok, (seed, capi.STRATEGY_NAMES[strategy], i, worst)
+    # gathered strips can only add to what the 16-row strips took, and every entry
+    # still has exactly one owner
+    natural = (st.mfma_tiles, st.nnz_mfma) if st.strategy_used != capi.FLAT else (0, 0)
+    monkeypatch.setenv("SDDMM_GATHERED", "1")
+    e.plan(capi.AUTO)
+    e.run()
+    st = e.stats()
+    if st.strategy_used != capi.FLAT:
+        assert st.mfma_tiles >= natural[0] and st.nnz_mfma >= natural[1]
+        assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
+    ok, worst, i = O.check_values(e.values(), ref, mag=mag)
+    assert ok, (seed, "AUTO with gathered strips", i, worst)
     e.close()
