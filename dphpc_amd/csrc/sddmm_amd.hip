@@ -87,6 +87,7 @@ struct sddmm_ctx {
     RowItem *d_panel_items = nullptr;
     int64_t n_panel_items = 0, panel_items_cap = 0, n_panels = 0, nnz_panels = 0;
     bool panel_mfma = false;         // panels run on k_panel_mfma (else on k_panel)
+    bool panels_flagged = false;     // the panel detector ran in this plan
 };
 
 namespace {
@@ -458,18 +459,21 @@ int plan_tiles_count(sddmm_ctx *c, int min_fill) {
     hipLaunchKernelGGL(k_strip_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
                        c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner, c->d_pc);
     HIP_TRY(c, hipGetLastError());
-    int rc = device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
-    if (rc) return rc;
-    rc = fetch_counters(c);
-    if (rc) return rc;
+    return device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
+}
+
+// after a fetch_counters that follows plan_tiles_count (and precedes the gathered strips)
+int take_tile_counts(sddmm_ctx *c) {
     c->n_tiles = c->n_tiles_natural = (int64_t)c->pc.n_tiles;
     c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
-    if ((int64_t)c->pc.tiles_scanned != c->n_tiles)
+    if (c->tile_steps != 0 && (int64_t)c->pc.tiles_scanned != c->n_tiles)
         return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
     return SDDMM_OK;
 }
 
-int plan_gathered_count(sddmm_ctx *c, int min_fill, int min_len) {
+// Candidates of the gathered strips (launch only; the count arrives with the next
+// fetch_counters).
+int plan_gathered_candidates(sddmm_ctx *c, int min_len) {
     if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
     const int64_t M = c->sM;
     if (M > c->cand_cap) {
@@ -484,10 +488,15 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill, int min_len) {
                        c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys, c->d_cand_rows,
                        &c->d_pc->n_candidates);
     HIP_TRY(c, hipGetLastError());
-    int rc = fetch_counters(c);
-    if (rc) return rc;
+    return SDDMM_OK;
+}
+
+// after the fetch_counters that follows plan_gathered_candidates
+int plan_gathered_count(sddmm_ctx *c, int min_fill) {
+    if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
     c->n_cand = (int64_t)c->raw.n_candidates;
     if (c->n_cand < 2) { c->n_cand = 0; return SDDMM_OK; }
+    int rc;
     // candidates ordered by first column (the append order of the candidates is not
     // deterministic, the sorted order of equal keys therefore is not either: only the
     // grouping into strips can differ between plans, never a result)
@@ -571,7 +580,9 @@ bool panel_valu_applicable(const sddmm_ctx *c) {
     return s.unit == 0 ? s.UPL <= 2 : s.UPL == 1;
 }
 
-int plan_panels(sddmm_ctx *c, int min_len, int pseg) {
+// panel detector (launch only) / panel items (after the next fetch_counters)
+int plan_panels_flags(sddmm_ctx *c, int min_len, int pseg) {
+    c->panels_flagged = false;
     if (c->nnz == 0) return SDDMM_OK;
     c->panel_mfma = panel_mfma_steps(c) != 0 && env_int("SDDMM_PANEL_MFMA", 1) != 0;
     if (!c->panel_mfma && !panel_valu_applicable(c)) return SDDMM_OK;
@@ -588,10 +599,13 @@ int plan_panels(sddmm_ctx *c, int min_len, int pseg) {
     hipLaunchKernelGGL(k_panel_flags, dim3((unsigned)((n_panels * WAVE + 255) / 256)), dim3(256), 0, c->stream,
                        c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner, c->d_panel_counts, c->d_pc);
     HIP_TRY(c, hipGetLastError());
-    int rc = device_scan(c, c->d_panel_counts, c->d_panel_off, n_panels, &c->d_pc->panel_items);
-    if (rc) return rc;
-    rc = fetch_counters(c);
-    if (rc) return rc;
+    c->panels_flagged = true;
+    return device_scan(c, c->d_panel_counts, c->d_panel_off, n_panels, &c->d_pc->panel_items);
+}
+
+int plan_panels_items(sddmm_ctx *c, int pseg) {
+    if (!c->panels_flagged) return SDDMM_OK;
+    const int64_t n_panels = (int64_t)c->sM / 8;
     c->n_panels = (int64_t)c->pc.n_panels;
     c->nnz_panels = (int64_t)c->pc.nnz_panels;
     c->n_panel_items = (int64_t)c->pc.panel_items;
@@ -782,6 +796,10 @@ int do_plan(sddmm_ctx *c, int strategy) {
             // and 512 bytes; 64-byte rows keep the older, conservative figure
             const size_t row_bytes = (size_t)c->K * elem_size(c->dtype);
             const int tile_fill = std::max(1, env_int("SDDMM_TILE_FILL", row_bytes <= 64 ? 96 : row_bytes <= 128 ? 80 : 56));
+            const int pseg = std::max(WAVE, env_int("SDDMM_PANEL_SEG", 512));
+            const bool gathered = resolved == SDDMM_AUTO && env_int("SDDMM_GATHERED", 1) != 0;
+            c->tile_steps = 0;
+            // the classifiers are launched back to back; their totals come back together
             if (resolved != SDDMM_LDS_TILED) {
                 // 16-row strips are looked at before the row panels and must not take what the
                 // panel kernel does better (8x8-block rows reach ~80 entries per tile); the
@@ -790,13 +808,23 @@ int do_plan(sddmm_ctx *c, int strategy) {
                 if (rc) return rc;
             }
             if (resolved != SDDMM_MFMA_TILE) {
-                rc = plan_panels(c, resolved == SDDMM_LDS_TILED ? 1 : std::max(1, env_int("SDDMM_PANEL_MIN", 16)),
-                                 std::max(WAVE, env_int("SDDMM_PANEL_SEG", 512)));
+                rc = plan_panels_flags(c, resolved == SDDMM_LDS_TILED ? 1 : std::max(1, env_int("SDDMM_PANEL_MIN", 16)), pseg);
+                if (rc) return rc;
+            } else {
+                c->panels_flagged = false;
+            }
+            if (gathered) {
+                rc = plan_gathered_candidates(c, std::max(16, env_int("SDDMM_GATHERED_MIN", 64)));
                 if (rc) return rc;
             }
-            if (resolved == SDDMM_AUTO && env_int("SDDMM_GATHERED", 1) != 0) {
-                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)),
-                                         std::max(16, env_int("SDDMM_GATHERED_MIN", 64)));
+            rc = fetch_counters(c);
+            if (rc) return rc;
+            rc = take_tile_counts(c);
+            if (rc) return rc;
+            rc = plan_panels_items(c, pseg);
+            if (rc) return rc;
+            if (gathered) {
+                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)));
                 if (rc) return rc;
             }
             if (resolved != SDDMM_LDS_TILED) {
