@@ -593,3 +593,55 @@ def test_row_panels(engine_factory, monkeypatch, K, dtype):
     assert (st.panels == 5) == valu_applicable and (st.panels == 0) == (not valu_applicable)
     flat, _ = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.FLAT, dt)
     np.testing.assert_array_equal(flat.view(np.uint32), lds.view(np.uint32))
+
+
+@pytest.mark.parametrize("K,dtype", [(32, "f32"), (128, "f32"), (64, "bf16"), (256, "f16")])
+def test_gathered_strips(engine_factory, monkeypatch, K, dtype):
+    """Near-dense rows scattered over S: no 16 consecutive rows share tiles, but the
+    rows sorted by their first column do.  Ties in the first column, a candidate count
+    that is not a multiple of 16, one unsorted candidate and rows too short or too
+    spread out to be candidates are all in the mix."""
+    rng = np.random.default_rng(400 + K)
+    M, N = 1000, 5000
+    rows = [np.sort(rng.choice(N, int(rng.integers(1, 12)), replace=False)) for _ in range(M)]
+    dense_rows = np.sort(rng.choice(M, 203, replace=False))               # 203 = 12 strips of 16 + 11
+    starts = rng.choice([100, 100, 100, 900, 2500, 2500, 4000], len(dense_rows))   # many equal first columns
+    for r, s0 in zip(dense_rows, starts):
+        c = s0 + np.nonzero(rng.random(400) < 0.6)[0]
+        c[0] = s0                                                          # the first column itself: ties
+        rows[r] = np.unique(c)
+    spread = [int(x) for x in rng.choice(np.setdiff1d(np.arange(M), dense_rows), 20, replace=False)]
+    for r in spread:                                                       # long but not compact: no candidates
+        rows[r] = np.sort(rng.choice(N, 200, replace=False))
+    bad = int(dense_rows[7])
+    rows[bad] = np.concatenate([rows[bad][:5], rows[bad][5:7][::-1], rows[bad][7:]])   # one candidate is not sorted
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == "bf16":
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B, ops, dt = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K), (Ab, Bb), capi.BF16
+    elif dtype == "f16":
+        Ab, Bb = capi.to_f16(A).reshape(M, K), capi.to_f16(B).reshape(N, K)
+        A, B, ops, dt = capi.from_f16(Ab).reshape(M, K), capi.from_f16(Bb).reshape(N, K), (Ab, Bb), capi.F16
+    else:
+        ops, dt = (A, B), capi.F32
+    got, st = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert_parity(got, rowptr, col, val, A, B, what="gathered strips")
+    dense_nnz = int(lens[dense_rows].sum())
+    # of the 13 strips, the one with the unsorted row and up to three that straddle two
+    # windows (too few entries per tile) may be given up
+    assert st.mfma_tiles > 0 and 0.6 * dense_nnz <= st.nnz_mfma <= dense_nnz
+    assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
+    assert st.kernels_launched == 1
+    monkeypatch.setenv("SDDMM_FUSE", "0")
+    two, st2 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st2.kernels_launched == 2 and st2.nnz_mfma <= dense_nnz
+    assert_parity(two, rowptr, col, val, A, B, what="gathered strips, two launches")
+    monkeypatch.setenv("SDDMM_GATHERED", "0")
+    off, st3 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st3.mfma_tiles == 0
+    assert_parity(off, rowptr, col, val, A, B, what="gathered strips off")
