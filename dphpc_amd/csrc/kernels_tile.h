@@ -352,7 +352,8 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
 // Rows that are dense inside a column window need not be neighbours to share tiles:
 // any 16 rows whose windows overlap form a strip for the matrix cores as well as 16
 // consecutive ones do.  Candidate rows (not owned yet, at least min_len entries that
-// fill a quarter of their column span or more) are sorted by their first column;
+// fill a quarter of their column span or more) are sorted by (first column, row) --
+// one 64-bit key per row, so the order does not depend on the order of the appends;
 // every 16 consecutive rows of that order are one gathered strip, classified with
 // the same bitmap and threshold as a natural strip.  TileDesc.strip of such a strip
 // is GATHERED_BASE + its index, its rows are listed in a table (16 per strip, -1 for
@@ -362,7 +363,7 @@ constexpr int GATHERED_BASE = 1 << 30;
 __global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__restrict__ rowptr,
                                                            const int32_t *__restrict__ col, int M,
                                                            const unsigned char *__restrict__ owner, int min_len,
-                                                           unsigned int *__restrict__ keys, int32_t *__restrict__ rows,
+                                                           unsigned long long *__restrict__ keys,
                                                            unsigned long long *__restrict__ count) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     bool cand = false;
@@ -385,8 +386,7 @@ __global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__rest
            (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
     if (cand) {
         const unsigned long long at = base + (unsigned long long)__popcll(m & ((1ull << lane) - 1ull));
-        keys[at] = (unsigned int)first;
-        rows[at] = (int32_t)r;
+        keys[at] = ((unsigned long long)(unsigned int)first << 32) | (unsigned long long)(unsigned int)r;
     }
 }
 
@@ -398,12 +398,12 @@ struct GatheredHead {
 };
 __device__ __forceinline__ GatheredHead gathered_head(const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
-                                                      const int32_t *__restrict__ sorted_rows, int64_t n_cand,
-                                                      int64_t vs) {
+                                                      const unsigned long long *__restrict__ sorted_keys,
+                                                      int64_t n_cand, int64_t vs) {
     GatheredHead h;
     const int lane = lane_id();
     const int64_t idx = vs * 16 + lane;
-    h.row = lane < 16 && idx < n_cand ? sorted_rows[idx] : -1;
+    h.row = lane < 16 && idx < n_cand ? (int)(unsigned int)sorted_keys[idx] : -1;   // low half of the key
     h.s = h.row >= 0 ? rowptr[h.row] : 0;
     h.e = h.row >= 0 ? rowptr[h.row + 1] : 0;
     const bool has = h.e > h.s;
@@ -439,7 +439,8 @@ __device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, c
 // pass 1 of the gathered strips: tiles per strip (0: not taken), the strip's row
 // table, ownership of the rows of a taken strip.
 __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_count(
-    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, const int32_t *__restrict__ sorted_rows,
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
+    const unsigned long long *__restrict__ sorted_keys,
     int64_t n_cand, int64_t n_vstrips, int min_fill, unsigned int *__restrict__ vstrip_ntiles,
     int32_t *__restrict__ vrows, unsigned char *__restrict__ owner, DevCounters *pc) {
     __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
@@ -447,7 +448,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_count(
     if (vs >= n_vstrips) return;
     unsigned int *bm = bm_all[wave_in_block()];
     const int lane = lane_id();
-    const GatheredHead h = gathered_head(rowptr, col, sorted_rows, n_cand, vs);
+    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);
     if (lane < 16) vrows[vs * 16 + lane] = h.row;
     int64_t tiles = 0;
     bool take = false;
@@ -471,7 +472,8 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_count(
 
 // pass 2 of the gathered strips: strip and tile column of every descriptor
 __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_tiles(
-    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, const int32_t *__restrict__ sorted_rows,
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
+    const unsigned long long *__restrict__ sorted_keys,
     int64_t n_cand, int64_t n_vstrips, const unsigned int *__restrict__ vstrip_ntiles,
     const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles) {
     __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
@@ -480,7 +482,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_tiles(
     if (vstrip_ntiles[vs] == 0) return;
     unsigned int *bm = bm_all[wave_in_block()];
     const int lane = lane_id();
-    const GatheredHead h = gathered_head(rowptr, col, sorted_rows, n_cand, vs);
+    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);
     (void)gathered_mark(col, h, bm);
     const int words = (h.span + 31) >> 5;
     int64_t run = vstrip_off[vs];

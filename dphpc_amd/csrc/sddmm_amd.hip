@@ -71,8 +71,8 @@ struct sddmm_ctx {
     bool tiles_active = false;       // d_tiles describes the current pattern
     int64_t n_tiles_natural = 0;     // descriptors of 16-row strips come first, gathered strips after
     // gathered strips: candidate rows, sorted by first column, 16 per strip
-    unsigned int *d_cand_keys = nullptr, *d_sorted_keys = nullptr;
-    int32_t *d_cand_rows = nullptr, *d_sorted_rows = nullptr, *d_vrows = nullptr;
+    unsigned long long *d_cand_keys = nullptr, *d_sorted_keys = nullptr;   // (first column << 32) | row
+    int32_t *d_vrows = nullptr;
     void *d_sort_tmp = nullptr;
     size_t sort_tmp_bytes = 0;
     int64_t cand_cap = 0, vstrips_cap = 0, n_cand = 0, n_vstrips = 0;
@@ -144,7 +144,7 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_strip_ntiles);
     dfree(c->d_strip_off);
     dfree(c->d_tiles);
-    dfree(c->d_cand_keys); dfree(c->d_sorted_keys); dfree(c->d_cand_rows); dfree(c->d_sorted_rows);
+    dfree(c->d_cand_keys); dfree(c->d_sorted_keys);
     dfree(c->d_vrows); dfree(c->d_sort_tmp); dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off);
     c->sort_tmp_bytes = 0;
     c->cand_cap = c->vstrips_cap = c->n_cand = c->n_vstrips = 0;
@@ -477,15 +477,13 @@ int plan_gathered_candidates(sddmm_ctx *c, int min_len) {
     if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
     const int64_t M = c->sM;
     if (M > c->cand_cap) {
-        dfree(c->d_cand_keys); dfree(c->d_sorted_keys); dfree(c->d_cand_rows); dfree(c->d_sorted_rows);
-        ALLOC_TRY(c, c->d_cand_keys, (size_t)M * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_sorted_keys, (size_t)M * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_cand_rows, (size_t)M * sizeof(int32_t));
-        ALLOC_TRY(c, c->d_sorted_rows, (size_t)M * sizeof(int32_t));
+        dfree(c->d_cand_keys); dfree(c->d_sorted_keys);
+        ALLOC_TRY(c, c->d_cand_keys, (size_t)M * sizeof(unsigned long long));
+        ALLOC_TRY(c, c->d_sorted_keys, (size_t)M * sizeof(unsigned long long));
         c->cand_cap = M;
     }
     hipLaunchKernelGGL(k_gather_candidates, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, c->stream, c->d_rowptr,
-                       c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys, c->d_cand_rows,
+                       c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys,
                        &c->d_pc->n_candidates);
     HIP_TRY(c, hipGetLastError());
     return SDDMM_OK;
@@ -497,19 +495,17 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
     c->n_cand = (int64_t)c->raw.n_candidates;
     if (c->n_cand < 2) { c->n_cand = 0; return SDDMM_OK; }
     int rc;
-    // candidates ordered by first column (the append order of the candidates is not
-    // deterministic, the sorted order of equal keys therefore is not either: only the
-    // grouping into strips can differ between plans, never a result)
+    // candidates ordered by (first column, row)
     size_t need = 0;
-    HIP_TRY(c, rocprim::radix_sort_pairs(nullptr, need, c->d_cand_keys, c->d_sorted_keys, c->d_cand_rows,
-                                         c->d_sorted_rows, (size_t)c->n_cand, 0, 32, c->stream));
+    HIP_TRY(c, rocprim::radix_sort_keys(nullptr, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
+                                        c->stream));
     if (need > c->sort_tmp_bytes) {
         dfree(c->d_sort_tmp);
         ALLOC_TRY(c, c->d_sort_tmp, need);
         c->sort_tmp_bytes = need;
     }
-    HIP_TRY(c, rocprim::radix_sort_pairs(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, c->d_cand_rows,
-                                         c->d_sorted_rows, (size_t)c->n_cand, 0, 32, c->stream));
+    HIP_TRY(c, rocprim::radix_sort_keys(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
+                                        c->stream));
     c->n_vstrips = (c->n_cand + 15) / 16;
     if (c->n_vstrips > c->vstrips_cap) {
         dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off); dfree(c->d_vrows);
@@ -520,7 +516,7 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
     }
     const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
     hipLaunchKernelGGL(k_gathered_count, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr, c->d_col,
-                       (const int32_t *)c->d_sorted_rows, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
+                       (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
                        c->d_vrows, c->d_owner, c->d_pc);
     HIP_TRY(c, hipGetLastError());
     rc = device_scan(c, c->d_vstrip_ntiles, c->d_vstrip_off, c->n_vstrips, &c->d_pc->tiles_scanned);
@@ -551,7 +547,7 @@ int plan_tiles_fill(sddmm_ctx *c) {
     if (c->n_tiles > c->n_tiles_natural) {
         const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
         hipLaunchKernelGGL(k_gathered_tiles, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
-                           c->d_col, (const int32_t *)c->d_sorted_rows, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
+                           c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
                            c->d_vstrip_off, c->d_tiles + c->n_tiles_natural);
         HIP_TRY(c, hipGetLastError());
     }
