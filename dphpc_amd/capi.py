@@ -24,7 +24,8 @@ EXPORTS = [
     "sddmm_create", "sddmm_destroy", "sddmm_strerror", "sddmm_last_error",
     "sddmm_set_dense", "sddmm_set_dense_device", "sddmm_set_csr", "sddmm_set_coo",
     "sddmm_set_csr_device", "sddmm_update_values", "sddmm_plan", "sddmm_run",
-    "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_get_values",
+    "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_run_fused",
+    "sddmm_get_fused", "sddmm_get_fused_device", "sddmm_get_values",
     "sddmm_get_values_device", "sddmm_last_stats", "sddmm_partition_rows", "sddmm_version",
 ]
 
@@ -87,6 +88,9 @@ def load_library():
     L.sddmm_synchronize.argtypes = [vp]
     L.sddmm_time_runs.argtypes = [vp, i32, i32, i32, vp]
     L.sddmm_time_region.argtypes = [vp, i32, i32, C.POINTER(C.c_float)]
+    L.sddmm_run_fused.argtypes = [vp]
+    L.sddmm_get_fused.argtypes = [vp, vp]
+    L.sddmm_get_fused_device.argtypes = [vp, C.POINTER(vp)]
     L.sddmm_get_values.argtypes = [vp, vp]
     L.sddmm_get_values_device.argtypes = [vp, C.POINTER(vp)]
     L.sddmm_last_stats.argtypes = [vp, C.POINTER(Stats)]
@@ -174,6 +178,7 @@ class Engine:
             B = np.ascontiguousarray(B, np.uint16)
         assert A.ndim == 2 and B.ndim == 2 and A.shape[1] == B.shape[1]
         self._chk(self.L.sddmm_set_dense(self.h, A.shape[0], B.shape[0], A.shape[1], _ptr(A), _ptr(B), dtype))
+        self._dense_shape = (A.shape[0], A.shape[1])
 
     def set_csr(self, M, N, rowptr, col, sval):
         rowptr = np.ascontiguousarray(rowptr, np.int32)
@@ -216,6 +221,13 @@ class Engine:
         total = C.c_float(0.0)
         self._chk(self.L.sddmm_time_region(self.h, reps, int(include_plan), C.byref(total)))
         return float(total.value)
+
+    def run_fused(self):
+        """SDDMM followed by SpMM over the same pattern; returns O (M x K, fp32)."""
+        self._chk(self.L.sddmm_run_fused(self.h))
+        O = np.empty(self._dense_shape, np.float32)
+        self._chk(self.L.sddmm_get_fused(self.h, _ptr(O)))
+        return O
 
     def values(self):
         P = np.empty(self.nnz, np.float32)

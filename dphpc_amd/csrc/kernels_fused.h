@@ -1,0 +1,129 @@
+// SDDMM followed by SpMM over the same pattern ("FusedMM"):
+//
+//     P[i,j] = S[i,j] * <A[i,:], B[j,:]>          (what the SDDMM kernels compute)
+//     O[i,:] = sum over stored (i,j) of P[i,j] * B[j,:]
+//
+// The step that consumes an SDDMM result in the applications the reference names
+// (attention-like updates in graph learning); the reference itself stops at P.
+// The gathered B row of an entry is used twice while it sits in registers, so the
+// second product costs no memory traffic beyond the M x K output.
+//
+// One wavefront per work item = entries [start,end) of one row, in the lane layout
+// of the gather kernels: groups of LPN lanes, lane j of a group holds units
+// j, j+LPN, ... of the A row, of the entry's B row and of the group's partial output
+// row.  After the last entry the partial rows of the 64/LPN groups are added with
+// lane permutes; group 0 writes the output row, or adds it atomically when the row
+// was split into several items (O is cleared before the launch).
+#pragma once
+#include "kernels_gather.h"
+
+namespace sddmm {
+
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                   const int32_t *__restrict__ rowptr,
+                                                   const int32_t *__restrict__ col,
+                                                   const float *__restrict__ sval, float *__restrict__ P,
+                                                   float *__restrict__ O, const RowItem *__restrict__ items,
+                                                   int64_t n_items, int64_t nblocks) {
+    using U = typename L::U;
+    using T = typename U::T;                          // float4
+    using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
+    using Off_t = typename C::O;
+    constexpr int LPN = L::LPN, UPL = L::UPL, G = WAVE / LPN;
+    constexpr int NB = C::BIG;                        // steps whose gathers are in flight together
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t w = blk * WAVES_PER_BLOCK + wave_in_block();
+    if (w >= n_items) return;
+    const RowItem it = items[w];
+    const int row = __builtin_amdgcn_readfirstlane(it.row);
+    const int start = __builtin_amdgcn_readfirstlane(it.start);
+    const int end = __builtin_amdgcn_readfirstlane(it.end);
+    if (start >= end) return;
+    const int lane = lane_id();
+    const int g = lane / LPN, j = lane & (LPN - 1);
+    const Off_t rb = (Off_t)KU * (Off_t)sizeof(T);
+    const typename C::Areg a = C::load_a(A, (Off_t)row * rb, j, KU);
+    T acc[UPL];
+#pragma unroll
+    for (int i = 0; i < UPL; ++i) acc[i] = U::zero();
+    const int last = end - 1;
+    for (int base = start; base < end; base += WAVE) {
+        const int n = base + lane;
+        const bool valid = n < end;
+        const int c = col[n < last ? n : last];
+        const float s = valid ? sval[n] : 0.f;        // entries past the end contribute p = 0
+        const Off_t boff = (Off_t)c * rb;
+        const int count = end - base < WAVE ? end - base : WAVE;
+        int steps = (count + G - 1) / G;
+        steps = steps < LPN ? steps : LPN;
+        float out = 0.f;
+        for (int t0 = 0; t0 < steps; t0 += NB) {
+            T bf[NB][UPL];
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const int src = ((t0 + q) * G + g) & (WAVE - 1);
+                const Off_t bo = shfl_off<Off_t>(boff, src);
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
+                    bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                if (t0 + q >= steps) break;               // wave-uniform
+                const int src = ((t0 + q) * G + g) & (WAVE - 1);
+                float p = 0.f;
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const float d = U::dot(a.u[i], bf[q][i], p);
+                    p = C::unit_on(j, i, KU) ? d : p;
+                }
+                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    acc[i].x = __builtin_fmaf(p, bf[q][i].x, acc[i].x);
+                    acc[i].y = __builtin_fmaf(p, bf[q][i].y, acc[i].y);
+                    acc[i].z = __builtin_fmaf(p, bf[q][i].z, acc[i].z);
+                    acc[i].w = __builtin_fmaf(p, bf[q][i].w, acc[i].w);
+                }
+                if (j == t0 + q) out = p;
+            }
+        }
+        // entry l = t*G+g was kept by lane g*LPN+t
+        const float res = __shfl(out, (lane % G) * LPN + lane / G, WAVE);
+        if (valid) P[n] = res;
+    }
+    // add the partial output rows of the G groups: lanes with the same j
+#pragma unroll
+    for (int off = LPN; off < WAVE; off <<= 1) {
+#pragma unroll
+        for (int i = 0; i < UPL; ++i) {
+            acc[i].x += __shfl_xor(acc[i].x, off, WAVE);
+            acc[i].y += __shfl_xor(acc[i].y, off, WAVE);
+            acc[i].z += __shfl_xor(acc[i].z, off, WAVE);
+            acc[i].w += __shfl_xor(acc[i].w, off, WAVE);
+        }
+    }
+    if (g == 0) {
+        const bool whole_row = start == rowptr[row] && end == rowptr[row + 1];
+        float *orow = O + (int64_t)row * KU * 4;
+#pragma unroll
+        for (int i = 0; i < UPL; ++i) {
+            const int u = j + i * LPN;
+            if (!C::unit_on(j, i, KU)) continue;
+            if (whole_row) {
+                *reinterpret_cast<T *>(orow + 4 * u) = acc[i];
+            } else {
+                atomicAdd(orow + 4 * u + 0, acc[i].x);
+                atomicAdd(orow + 4 * u + 1, acc[i].y);
+                atomicAdd(orow + 4 * u + 2, acc[i].z);
+                atomicAdd(orow + 4 * u + 3, acc[i].w);
+            }
+        }
+    }
+}
+
+}  // namespace sddmm

@@ -17,6 +17,7 @@
 #include <new>
 #include <vector>
 
+#include "kernels_fused.h"
 #include "kernels_gather.h"
 #include "kernels_plan.h"
 #include "kernels_tile.h"
@@ -88,6 +89,13 @@ struct sddmm_ctx {
     int64_t n_panel_items = 0, panel_items_cap = 0, n_panels = 0, nnz_panels = 0;
     bool panel_mfma = false;         // panels run on k_panel_mfma (else on k_panel)
     bool panels_flagged = false;     // the panel detector ran in this plan
+    // fused SDDMM + SpMM: items covering every non-empty row, output M x K
+    RowItem *d_fused_items = nullptr;
+    int64_t n_fused_items = 0, fused_items_cap = 0;
+    bool fused_items_valid = false;
+    float *dO = nullptr;
+    size_t o_cap = 0;
+    bool have_fused = false;
 };
 
 namespace {
@@ -129,6 +137,7 @@ void dfree(T *&p) {
 void release_dense(sddmm_ctx *c) {
     if (c->own_dense) { dfree(c->dA); dfree(c->dB); }
     c->dA = c->dB = nullptr;
+    c->have_fused = false;
     c->own_dense = false;
     c->have_dense = false;
     c->planned = false;
@@ -152,6 +161,9 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_panel_counts);
     dfree(c->d_panel_off);
     dfree(c->d_panel_items);
+    dfree(c->d_fused_items);
+    c->n_fused_items = c->fused_items_cap = 0;
+    c->fused_items_valid = c->have_fused = false;
     c->owner_cap = c->panels_cap = c->panel_items_cap = 0;
     c->n_panel_items = c->n_panels = c->nnz_panels = 0;
     c->owner_active = false;
@@ -932,6 +944,7 @@ void sddmm_destroy(sddmm_ctx *c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     release_dense(c);
     release_sparse(c);
+    dfree(c->dO);
     dfree(c->d_pc);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
@@ -1158,6 +1171,105 @@ int sddmm_run(sddmm_ctx *c) {
     HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
     c->stats.run_ms = ms;
     c->stats.kernels_launched = c->launches;
+    return SDDMM_OK;
+}
+
+// items of the fused kernel: every non-empty row, cut into segments of SDDMM_SEG entries
+static int plan_fused_items(sddmm_ctx *c) {
+    if (c->fused_items_valid) return SDDMM_OK;
+    const int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+    const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
+    if (nb > c->block_sums_cap) {
+        dfree(c->d_block_sums);
+        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
+        c->block_sums_cap = nb;
+    }
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
+                              sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
+    c->n_fused_items = 0;
+    if (nb > 0) {
+        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+                           (const unsigned char *)nullptr, c->sM, 1, seg, c->d_block_sums, c->d_pc);
+        hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
+                           &c->d_pc->n_items);
+        HIP_TRY(c, hipGetLastError());
+        DevCounters tmp;
+        HIP_TRY(c, hipMemcpyAsync(&tmp, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
+        HIP_TRY(c, hipStreamSynchronize(c->stream));
+        c->n_fused_items = (int64_t)tmp.n_items;
+        if (c->n_fused_items > c->fused_items_cap) {
+            dfree(c->d_fused_items);
+            ALLOC_TRY(c, c->d_fused_items, (size_t)c->n_fused_items * sizeof(RowItem));
+            c->fused_items_cap = c->n_fused_items;
+        }
+        if (c->n_fused_items > 0) {
+            hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+                               (const unsigned char *)nullptr, c->sM, 1, seg, c->d_block_sums, c->d_fused_items);
+            HIP_TRY(c, hipGetLastError());
+        }
+    }
+    c->fused_items_valid = true;
+    return SDDMM_OK;
+}
+
+int sddmm_run_fused(sddmm_ctx *c) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    int rc = check_ready(c);
+    if (rc) return rc;
+    const Shape s = shape_of(c);
+    if (c->dtype != SDDMM_F32 || s.unit != 0 || s.LPN == 0 || s.LPN > 8)
+        return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs fp32 operands with K a multiple of 4, K <= 256");
+    if (!c->have_rowptr) return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs row-sorted entries");
+    rc = plan_fused_items(c);
+    if (rc) return rc;
+    const size_t o_bytes = (size_t)c->M * (size_t)c->K * sizeof(float);
+    if (o_bytes > c->o_cap) {
+        dfree(c->dO);
+        c->o_cap = 0;
+        ALLOC_TRY(c, c->dO, o_bytes);
+        c->o_cap = o_bytes;
+    }
+    HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
+    if (o_bytes) HIP_TRY(c, hipMemsetAsync(c->dO, 0, o_bytes, c->stream));
+    if (c->n_fused_items > 0) {
+        const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+        with_layout(s, [&](auto L) {
+            using LT = decltype(L);
+            if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS == 4) {
+                hipLaunchKernelGGL((k_fusedmm<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                                   (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
+                                   c->dP, c->dO, (const RowItem *)c->d_fused_items, c->n_fused_items, nblocks);
+            }
+        });
+        HIP_TRY(c, hipGetLastError());
+    }
+    HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
+    HIP_TRY(c, hipEventSynchronize(c->ev1));
+    float ms = 0.f;
+    HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
+    c->stats.run_ms = ms;
+    c->stats.kernels_launched = c->n_fused_items > 0 ? 1 : 0;
+    c->have_fused = true;
+    return SDDMM_OK;
+}
+
+int sddmm_get_fused(sddmm_ctx *c, float *O) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    if (!c->have_fused) return fail(c, SDDMM_ERR_STATE, "no fused result: call sddmm_run_fused first");
+    const size_t o_bytes = (size_t)c->M * (size_t)c->K * sizeof(float);
+    if (o_bytes > 0 && !O) return fail(c, SDDMM_ERR_NULL, "O is NULL");
+    if (o_bytes) HIP_TRY(c, hipMemcpyAsync(O, c->dO, o_bytes, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    return SDDMM_OK;
+}
+
+int sddmm_get_fused_device(sddmm_ctx *c, const float **dO) {
+    if (!c || !dO) return SDDMM_ERR_NULL;
+    if (!c->have_fused) return fail(c, SDDMM_ERR_STATE, "no fused result: call sddmm_run_fused first");
+    *dO = c->dO;
     return SDDMM_OK;
 }
 

@@ -155,6 +155,19 @@ int sddmm_time_runs(sddmm_ctx *ctx, int warmup, int reps, int include_plan, floa
  * per-launch synchronisation of sddmm_time_runs puts in front of every launch. */
 int sddmm_time_region(sddmm_ctx *ctx, int reps, int include_plan, float *total_ms);
 
+/* ---- SDDMM followed by SpMM over the same pattern ("FusedMM") -------------- */
+/* O[i,:] = sum over the stored (i,j) of P[i,j] * B[j,:], with P as sddmm_run computes
+ * it (and written like it): the step that consumes an SDDMM result in the applications
+ * the reference names.  No counterpart in the reference's code, which stops at P
+ * (src/competitors/cpu/cpu_basic.hpp:18-51).  O is M x K fp32 row-major, owned by the
+ * context.  Needs fp32 operands with K a multiple of 4 and K <= 256, and row-sorted
+ * entries (CSR, or COO with non-decreasing rows); SDDMM_ERR_UNSUPPORTED otherwise.
+ * Rows longer than 2048 entries are accumulated with atomic adds, so their last bits
+ * may differ from run to run. */
+int sddmm_run_fused(sddmm_ctx *ctx);
+int sddmm_get_fused(sddmm_ctx *ctx, float *O);                    /* M*K floats to the host */
+int sddmm_get_fused_device(sddmm_ctx *ctx, const float **dO);     /* valid until the next set_* / destroy */
+
 /* ---- results (cleanup phase) -------------------------------------------- */
 /* nnz floats in the entry order of the input (pattern is never permuted). */
 int sddmm_get_values(sddmm_ctx *ctx, float *P_values);

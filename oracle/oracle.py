@@ -50,6 +50,10 @@ def lib():
         L.oracle_sddmm_coo_f32.restype = None
         L.oracle_sddmm_csr_f64.argtypes = [C.c_int, C.c_int, _i32p, _i32p, _f32p, _f32p, _f32p, _f64p, _f64p]
         L.oracle_sddmm_csr_f64.restype = None
+        L.oracle_fusedmm_csr_f32.argtypes = [C.c_int, C.c_int, _i32p, _i32p, _f32p, _f32p, _f32p, _f32p, _f32p]
+        L.oracle_fusedmm_csr_f32.restype = None
+        L.oracle_fusedmm_csr_f64.argtypes = [C.c_int, C.c_int, _i32p, _i32p, _f32p, _f32p, _f32p, _f64p, _f64p]
+        L.oracle_fusedmm_csr_f64.restype = None
         L.oracle_triplets_sort_unique.argtypes = [C.c_int64, _i32p, _i32p, _f32p]
         L.oracle_triplets_sort_unique.restype = C.c_int64
         L.oracle_csr_from_triplets.argtypes = [C.c_int, C.c_int64, _i32p, _i32p, _f32p, _i32p, _i32p, _f32p]
@@ -99,6 +103,28 @@ def sddmm_csr_f64(rowptr, col, sval, A, B):
     m = np.zeros(len(col), np.float64)
     lib().oracle_sddmm_csr_f64(len(rowptr) - 1, A.shape[1], rowptr, col, sval, A, B, d, m)
     return d, m
+
+
+def fusedmm_csr(rowptr, col, sval, A, B):
+    """(P, O): SDDMM values and O = P @ B over the same pattern, fp32 in storage order."""
+    rowptr, col, sval = _c(rowptr, np.int32), _c(col, np.int32), _c(sval, np.float32)
+    A, B = _c(A, np.float32), _c(B, np.float32)
+    M, K = len(rowptr) - 1, A.shape[1]
+    P = np.zeros(len(col), np.float32)
+    Out = np.zeros((M, K), np.float32)
+    lib().oracle_fusedmm_csr_f32(M, K, rowptr, col, sval, A, B, P, Out)
+    return P, Out
+
+
+def fusedmm_csr_f64(rowptr, col, sval, A, B):
+    """(O, magnitude) in double: error analysis / tolerance floor of the fused result."""
+    rowptr, col, sval = _c(rowptr, np.int32), _c(col, np.int32), _c(sval, np.float32)
+    A, B = _c(A, np.float32), _c(B, np.float32)
+    M, K = len(rowptr) - 1, A.shape[1]
+    o = np.zeros((M, K), np.float64)
+    m = np.zeros((M, K), np.float64)
+    lib().oracle_fusedmm_csr_f64(M, K, rowptr, col, sval, A, B, o, m)
+    return o, m
 
 
 def sddmm_csr_numpy(rowptr, col, sval, A, B):

@@ -18,6 +18,10 @@
  *   oracle_dispatch           matrices/CSR.hpp:196-264
  *   oracle_density            matrices/CSR.hpp:157-159 (in 64-bit; the reference
  *                             multiplies rows*cols in int and overflows above 46340^2)
+ *   oracle_fusedmm_csr_f32/_f64   no counterpart: the reference stops at P.  SpMM of
+ *                             the SDDMM result with B, written in the reference's
+ *                             style (multiply, then add, entries in storage order);
+ *                             pinned by numpy identities only (tests/test_oracle.py)
  *
  * Arithmetic contract of the reference loop: fp32 multiply, then fp32 add into
  * the running value, k ascending, then one fp32 multiply by the S value.  The
@@ -132,6 +136,54 @@ void oracle_sddmm_csr_f64(int M, int K,
             }
             if (dot64) dot64[j] = acc * (double)sval[j];
             if (mag64) mag64[j] = mag * fabs((double)sval[j]);
+        }
+    }
+}
+
+/* ---- SDDMM followed by SpMM over the same pattern (no counterpart) ------
+ * P as oracle_sddmm_csr_f32; O[i,:] = sum_j P[i,j] * B[col_j,:], fp32 multiply then
+ * fp32 add, entries in storage order. */
+void oracle_fusedmm_csr_f32(int M, int K,
+                            const int32_t *rowptr, const int32_t *col, const float *sval,
+                            const float *A, const float *B, float *P, float *O)
+{
+    oracle_sddmm_csr_f32(M, K, rowptr, col, sval, A, B, P);
+    for (int i = 0; i < M; i++) {
+        float *o = O + (size_t)i * (size_t)K;
+        for (int k = 0; k < K; k++) o[k] = 0.0f;
+        for (int32_t j = rowptr[i]; j < rowptr[i + 1]; j++) {
+            const float *b = B + (size_t)col[j] * (size_t)K;
+            for (int k = 0; k < K; k++)
+                o[k] += P[j] * b[k];
+        }
+    }
+}
+
+/* O64 = the same in double from the double SDDMM values; mag64[i,k] = sum_j
+ * |S_j| (sum_k' |a b|) |b_k|, the cancellation-free magnitude for a tolerance floor */
+void oracle_fusedmm_csr_f64(int M, int K,
+                            const int32_t *rowptr, const int32_t *col, const float *sval,
+                            const float *A, const float *B, double *O64, double *mag64)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int i = 0; i < M; i++) {
+        const float *a = A + (size_t)i * (size_t)K;
+        double *o = O64 + (size_t)i * (size_t)K, *m = mag64 + (size_t)i * (size_t)K;
+        for (int k = 0; k < K; k++) { o[k] = 0.0; m[k] = 0.0; }
+        for (int32_t j = rowptr[i]; j < rowptr[i + 1]; j++) {
+            const float *b = B + (size_t)col[j] * (size_t)K;
+            double acc = 0.0, mag = 0.0;
+            for (int k = 0; k < K; k++) {
+                double p = (double)a[k] * (double)b[k];
+                acc += p;
+                mag += fabs(p);
+            }
+            acc *= (double)sval[j];
+            mag *= fabs((double)sval[j]);
+            for (int k = 0; k < K; k++) {
+                o[k] += acc * (double)b[k];
+                m[k] += mag * fabs((double)b[k]);
+            }
         }
     }
 }

@@ -1,0 +1,110 @@
+"""SDDMM followed by SpMM over the same pattern (sddmm_run_fused) against the CPU
+oracle: O within 1e-5 of the fp32 storage-order result with the cancellation-free
+magnitude as floor, P to the bar of the SDDMM tests."""
+import numpy as np
+import pytest
+
+from dphpc_amd import capi, workloads as W
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def _check(e, rowptr, col, val, A, B, what):
+    got_o = e.run_fused()
+    got_p = e.values()
+    ref_p, ref_o = O.fusedmm_csr(rowptr, col, val, A, B)
+    _, mag_p = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    ok, worst, i = O.check_values(got_p, ref_p, mag=mag_p)
+    assert ok, "%s: P entry %d got %r ref %r (%.2f x tolerance)" % (what, i, got_p[i], ref_p[i], worst)
+    _, mag_o = O.fusedmm_csr_f64(rowptr, col, val, A, B)
+    M = len(rowptr) - 1
+    ok, worst, i = O.check_values(got_o[:M].ravel(), ref_o.ravel(), mag=mag_o.ravel())
+    assert ok, "%s: O element %d got %r ref %r (%.2f x tolerance)" % (what, i, got_o[:M].ravel()[i], ref_o.ravel()[i], worst)
+    assert not got_o[M:].any()                       # rows of A beyond S's rows stay zero
+    return got_o
+
+
+@pytest.mark.parametrize("K", [4, 8, 32, 48, 100, 128, 256])
+def test_fused_random(engine_factory, K):
+    rng = np.random.default_rng(900 + K)
+    M, N = 300, 260
+    dense = rng.random((M, N)) < 0.08
+    dense[17] = False
+    dense[40, :] = rng.random(N) < 0.9               # a long row
+    r, c = np.nonzero(dense)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    A = rng.uniform(-1, 1, (M + 3, K)).astype(f32)   # A may have more rows than S
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    out = _check(e, rowptr, col, val, A, B, "random K=%d" % K)
+    assert not out[17].any()
+    # repeatable, and the ordinary run still works on the same context
+    np.testing.assert_array_equal(out, e.run_fused())
+    e.plan(capi.AUTO); e.run()
+    ok, worst, i = O.check_values(e.values(), O.sddmm_csr(rowptr, col, val, A, B), mag=O.sddmm_csr_f64(rowptr, col, val, A, B)[1])
+    assert ok
+    e.close()
+
+
+def test_fused_rows_split_into_segments(engine_factory, monkeypatch):
+    """Rows longer than a segment are accumulated by several wavefronts (atomic adds)."""
+    monkeypatch.setenv("SDDMM_SEG", "128")
+    rng = np.random.default_rng(31)
+    M, N, K = 40, 3000, 32
+    rows = [np.sort(rng.choice(N, int(rng.choice([0, 5, 127, 128, 129, 700, 2500])), replace=False)) for _ in range(M)]
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    _check(e, rowptr, col, val, A, B, "segments")
+    e.close()
+
+
+@pytest.mark.parametrize("name", ["fem_banded", "power_law", "mixed_density"])
+def test_fused_benchmark_shapes_scaled_down(engine_factory, name):
+    w = W.make(name, "small")
+    e = engine_factory()
+    e.set_dense(w.A, w.B)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    _check(e, w.rowptr, w.col, w.sval, w.A, w.B, name)
+    # COO with sorted rows takes the same path
+    e.set_coo(w.M, w.N, w.rows(), w.col, w.sval)
+    _check(e, w.rowptr, w.col, w.sval, w.A, w.B, name + " coo")
+    e.close()
+
+
+def test_fused_unsupported_and_state(engine_factory):
+    rng = np.random.default_rng(3)
+    rowptr = np.array([0, 1, 2], np.int32); col = np.array([1, 0], np.int32); val = np.ones(2, f32)
+    e = engine_factory()
+    for K, dt in ((33, capi.F32), (260, capi.F32), (32, capi.BF16)):
+        A = rng.uniform(-1, 1, (2, K)).astype(f32)
+        if dt == capi.BF16:
+            e.set_dense(capi.to_bf16(A).reshape(2, K), capi.to_bf16(A).reshape(2, K), dt)
+        else:
+            e.set_dense(A, A)
+        e.set_csr(2, 2, rowptr, col, val)
+        with pytest.raises(capi.SddmmError) as ei:
+            e.run_fused()
+        assert ei.value.code == capi.ERR_UNSUPPORTED
+    A = rng.uniform(-1, 1, (2, 8)).astype(f32)
+    e.set_dense(A, A)
+    e.set_coo(2, 2, np.array([1, 0], np.int32), col, val)     # rows not sorted: no row pointer
+    with pytest.raises(capi.SddmmError) as ei:
+        e.run_fused()
+    assert ei.value.code == capi.ERR_UNSUPPORTED
+    e.set_csr(2, 2, rowptr, col, val)
+    out = e.run_fused()
+    want = np.stack([(A[0] @ A[1]) * A[1], (A[1] @ A[0]) * A[0]]).astype(f32)
+    np.testing.assert_allclose(out, want, rtol=1e-6, atol=1e-6)
+    e.close()

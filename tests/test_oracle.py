@@ -303,3 +303,45 @@ def test_comparator():
     assert ok                                         # 1e-7 <= 1e-5 * 0.25 * 1.0
     ok, _, _ = O.check_values(np.array([1.0, 2.0, 0.0, 1e-3], f32), ref, mag=mag)
     assert not ok                                     # sign error is caught (the reference's == would pass it)
+
+
+# ---- SDDMM followed by SpMM (no counterpart in the reference: pinned by identities) ----
+def test_fusedmm_oracle_against_dense_algebra():
+    """O = (S o (A B^T)) B.  Brute force in float64 on small inputs, the all-ones S
+    special case (O = A B^T B), a diagonal S (each output row is a multiple of one B
+    row), linearity in S, and the P half against the SDDMM oracle bit for bit."""
+    rng = np.random.default_rng(77)
+    M, N, K = 23, 17, 12
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (N, K)).astype(np.float32)
+    dense = rng.random((M, N)) < 0.4
+    dense[5, :] = False                                        # an empty row gives a zero output row
+    r, c = np.nonzero(dense)
+    v = rng.uniform(-1, 1, len(r)).astype(np.float32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    P, Out = O.fusedmm_csr(rowptr, col, val, A, B)
+    np.testing.assert_array_equal(P.view(np.uint32), O.sddmm_csr(rowptr, col, val, A, B).view(np.uint32))
+    S = np.zeros((M, N)); S[r, c] = v
+    want = (S * (A.astype(np.float64) @ B.astype(np.float64).T)) @ B.astype(np.float64)
+    np.testing.assert_allclose(Out, want, rtol=0, atol=2e-5)
+    assert not Out[5].any()
+    o64, mag = O.fusedmm_csr_f64(rowptr, col, val, A, B)
+    np.testing.assert_allclose(o64, want, rtol=1e-12, atol=1e-12)
+    assert (mag >= np.abs(o64) - 1e-12).all()
+    # all-ones S: plain matrix products
+    rr, cc = np.nonzero(np.ones((M, N), bool))
+    rp1, c1, v1 = O.csr_from_triplets(M, rr.astype(np.int32), cc.astype(np.int32), np.ones(len(rr), np.float32))
+    _, O1 = O.fusedmm_csr(rp1, c1, v1, A, B)
+    np.testing.assert_allclose(O1, A.astype(np.float64) @ B.astype(np.float64).T @ B.astype(np.float64), rtol=0, atol=5e-5)
+    # diagonal S: O[i] = s_i <a_i, b_i> b_i, three roundings
+    n = min(M, N)
+    d = np.arange(n, dtype=np.int32)
+    sv = rng.uniform(0.5, 2, n).astype(np.float32)
+    rpd, cd, vd = O.csr_from_triplets(M, d, d, sv)
+    Pd, Od = O.fusedmm_csr(rpd, cd, vd, A, B)
+    for i in range(n):
+        np.testing.assert_array_equal(Od[i], (Pd[i] * B[i]).astype(np.float32))
+    assert not Od[n:].any()
+    # linear in S, exactly for a factor 2
+    _, O2 = O.fusedmm_csr(rowptr, col, (val * np.float32(2)).astype(np.float32), A, B)
+    np.testing.assert_array_equal(O2, Out * np.float32(2))
