@@ -8,7 +8,8 @@
 // The gathered B row of an entry is used twice while it sits in registers, so the
 // second product costs no memory traffic beyond the M x K output.
 //
-// One wavefront per work item = entries [start,end) of one row, in the lane layout
+// k_fusedmm: one wavefront per work item = entries [start,end) of one row (rows longer
+// than FUSED_ROW_MAX entries; shorter ones go to k_fusedmm_rows), in the lane layout
 // of the gather kernels: groups of LPN lanes, lane j of a group holds units
 // j, j+LPN, ... of the A row, of the entry's B row and of the group's partial output
 // row.  After the last entry the partial rows of the 64/LPN groups are added with
@@ -18,6 +19,8 @@
 #include "kernels_gather.h"
 
 namespace sddmm {
+
+constexpr int FUSED_ROW_MAX = 64;   // rows up to this length: one row per lane group
 
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, const void *__restrict__ B, int KU,
@@ -122,6 +125,104 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
                 atomicAdd(orow + 4 * u + 2, acc[i].z);
                 atomicAdd(orow + 4 * u + 3, acc[i].w);
             }
+        }
+    }
+}
+
+// Rows of at most max_len entries, one row per lane group: a wavefront takes 64/LPN
+// consecutive rows, group g walks row r0+g.  Lane j of a group reads column index and
+// S value of entry t0+j, so LPN entries of each row are gathered back to back; the
+// P value of entry t0+j ends up in lane j, and the output row needs no reduction
+// across groups.  Longer rows are left to k_fusedmm (they count as empty here); every
+// other row, empty ones included, gets its output row written.
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                        const int32_t *__restrict__ rowptr,
+                                                        const int32_t *__restrict__ col,
+                                                        const float *__restrict__ sval, float *__restrict__ P,
+                                                        float *__restrict__ O, int M, int max_len, int64_t nblocks) {
+    using U = typename L::U;
+    using T = typename U::T;
+    using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
+    using Off_t = typename C::O;
+    constexpr int LPN = L::LPN, UPL = L::UPL, G = WAVE / LPN;
+    constexpr int NB = C::BIG;
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t r0 = (blk * WAVES_PER_BLOCK + wave_in_block()) * G;
+    if (r0 >= M) return;
+    const int lane = lane_id();
+    const int g = lane / LPN, j = lane & (LPN - 1);
+    const int64_t row = r0 + g;
+    int rs = 0, len = 0;
+    bool mine = false;
+    if (row < M) {
+        rs = rowptr[row];
+        len = rowptr[row + 1] - rs;
+        mine = len <= max_len;
+        if (!mine) len = 0;
+    }
+    int longest = len;
+    for (int off = LPN; off < WAVE; off <<= 1) {
+        const int o = __shfl_xor(longest, off, WAVE);
+        longest = o > longest ? o : longest;
+    }
+    longest = __builtin_amdgcn_readfirstlane(longest);
+    const Off_t rb = (Off_t)KU * (Off_t)sizeof(T);
+    const typename C::Areg a = C::load_a(A, (Off_t)(row < M ? row : 0) * rb, j, KU);
+    T acc[UPL];
+#pragma unroll
+    for (int i = 0; i < UPL; ++i) acc[i] = U::zero();
+    for (int t0 = 0; t0 < longest; t0 += LPN) {
+        const int e = t0 + j;
+        const bool has = e < len;
+        const int at = has ? rs + e : (len > 0 ? rs + len - 1 : 0);   // a valid position in every lane
+        const int c = col[at];
+        const float s = has ? sval[at] : 0.f;
+        const Off_t boff = (Off_t)c * rb;
+        const int steps = longest - t0 < LPN ? longest - t0 : LPN;
+        float out = 0.f;
+        for (int q0 = 0; q0 < steps; q0 += NB) {
+            T bf[NB][UPL];
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const int src = g * LPN + ((q0 + q) & (LPN - 1));
+                const Off_t bo = shfl_off<Off_t>(boff, src);
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
+                    bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                if (q0 + q >= steps) break;               // wave-uniform
+                const int src = g * LPN + ((q0 + q) & (LPN - 1));
+                float p = 0.f;
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const float d = U::dot(a.u[i], bf[q][i], p);
+                    p = C::unit_on(j, i, KU) ? d : p;
+                }
+                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    acc[i].x = __builtin_fmaf(p, bf[q][i].x, acc[i].x);
+                    acc[i].y = __builtin_fmaf(p, bf[q][i].y, acc[i].y);
+                    acc[i].z = __builtin_fmaf(p, bf[q][i].z, acc[i].z);
+                    acc[i].w = __builtin_fmaf(p, bf[q][i].w, acc[i].w);
+                }
+                if (j == q0 + q) out = p;
+            }
+        }
+        if (has) P[at] = out;
+    }
+    if (mine) {
+        float *orow = O + row * KU * 4;
+#pragma unroll
+        for (int i = 0; i < UPL; ++i) {
+            const int u = j + i * LPN;
+            if (C::unit_on(j, i, KU)) *reinterpret_cast<T *>(orow + 4 * u) = acc[i];
         }
     }
 }

@@ -1174,7 +1174,7 @@ int sddmm_run(sddmm_ctx *c) {
     return SDDMM_OK;
 }
 
-// items of the fused kernel: every non-empty row, cut into segments of SDDMM_SEG entries
+// items of the fused kernel: the rows of more than FUSED_ROW_MAX entries, cut into segments of SDDMM_SEG entries
 static int plan_fused_items(sddmm_ctx *c) {
     if (c->fused_items_valid) return SDDMM_OK;
     const int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
@@ -1190,7 +1190,7 @@ static int plan_fused_items(sddmm_ctx *c) {
     c->n_fused_items = 0;
     if (nb > 0) {
         hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
-                           (const unsigned char *)nullptr, c->sM, 1, seg, c->d_block_sums, c->d_pc);
+                           (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc);
         hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
         HIP_TRY(c, hipGetLastError());
@@ -1205,7 +1205,7 @@ static int plan_fused_items(sddmm_ctx *c) {
         }
         if (c->n_fused_items > 0) {
             hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
-                               (const unsigned char *)nullptr, c->sM, 1, seg, c->d_block_sums, c->d_fused_items);
+                               (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_fused_items);
             HIP_TRY(c, hipGetLastError());
         }
     }
@@ -1233,14 +1233,26 @@ int sddmm_run_fused(sddmm_ctx *c) {
     }
     HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
     if (o_bytes) HIP_TRY(c, hipMemsetAsync(c->dO, 0, o_bytes, c->stream));
-    if (c->n_fused_items > 0) {
-        const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    int launches = 0;
+    if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);
             if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS == 4) {
-                hipLaunchKernelGGL((k_fusedmm<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                const int64_t rows_per_wave = WAVE / LT::LPN;
+                const int64_t waves = ((int64_t)c->sM + rows_per_wave - 1) / rows_per_wave;
+                const int64_t rblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+                hipLaunchKernelGGL((k_fusedmm_rows<LT>), dim3((unsigned)xcd_grid(rblocks)), dim3(BLOCK), 0, c->stream,
                                    (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
-                                   c->dP, c->dO, (const RowItem *)c->d_fused_items, c->n_fused_items, nblocks);
+                                   c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks);
+                ++launches;
+                if (c->n_fused_items > 0) {
+                    const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+                    hipLaunchKernelGGL((k_fusedmm<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                                       (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col,
+                                       c->d_sval, c->dP, c->dO, (const RowItem *)c->d_fused_items, c->n_fused_items,
+                                       nblocks);
+                    ++launches;
+                }
             }
         });
         HIP_TRY(c, hipGetLastError());
@@ -1250,7 +1262,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
     float ms = 0.f;
     HIP_TRY(c, hipEventElapsedTime(&ms, c->ev0, c->ev1));
     c->stats.run_ms = ms;
-    c->stats.kernels_launched = c->n_fused_items > 0 ? 1 : 0;
+    c->stats.kernels_launched = launches;
     c->have_fused = true;
     return SDDMM_OK;
 }
