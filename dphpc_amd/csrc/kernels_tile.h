@@ -418,72 +418,84 @@ __device__ __forceinline__ GatheredHead gathered_head(const int32_t *__restrict_
     return h;
 }
 
-// marks the tile columns of the strip's 16 rows in bm; false when a row is not sorted
-__device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, const GatheredHead &h, unsigned int *bm) {
-    const int lane = lane_id();
+// One workgroup of 16 wavefronts per gathered strip: wave i streams row i of the
+// strip into the strip's tile-column bitmap in LDS (the rows are not neighbours in
+// the CSR arrays, so they are 16 independent streams).  Returns false when a row is
+// not sorted.  Every wave of the workgroup must call it.
+constexpr int GATHERED_BLOCK = 16 * WAVE;
+
+__device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, const GatheredHead &h, unsigned int *bm,
+                                              int *unsorted_flag) {
     const int words = (h.span + 31) >> 5;
-    for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
-    wave_lds_order();
-    bool sorted = true;
-    for (int i = 0; i < 16; ++i) {
-        const int si = __builtin_amdgcn_readlane(h.s, i), ei = __builtin_amdgcn_readlane(h.e, i);
-        if (ei <= si) continue;                  // wave-uniform
+    for (int w = (int)threadIdx.x; w < words; w += GATHERED_BLOCK) bm[w] = 0u;
+    if (threadIdx.x == 0) *unsorted_flag = 0;
+    __syncthreads();
+    const int wi = wave_in_block();
+    const int si = __builtin_amdgcn_readlane(h.s, wi), ei = __builtin_amdgcn_readlane(h.e, wi);
+    if (ei > si) {                                   // wave-uniform
         int64_t descents = 0;
         (void)strip_scan<true>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
-        sorted = sorted && descents == 0;
+        if (descents != 0 && lane_id() == 0) atomicOr(unsorted_flag, 1);
     }
-    wave_lds_order();
-    return sorted;
+    __syncthreads();
+    return *unsorted_flag == 0;
 }
 
 // pass 1 of the gathered strips: tiles per strip (0: not taken), the strip's row
 // table, ownership of the rows of a taken strip.
-__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_count(
+__global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_count(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
     const unsigned long long *__restrict__ sorted_keys,
     int64_t n_cand, int64_t n_vstrips, int min_fill, unsigned int *__restrict__ vstrip_ntiles,
     int32_t *__restrict__ vrows, unsigned char *__restrict__ owner, DevCounters *pc) {
-    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
-    const int64_t vs = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
-    if (vs >= n_vstrips) return;
-    unsigned int *bm = bm_all[wave_in_block()];
+    __shared__ unsigned int bm[STRIP_BM_WORDS];
+    __shared__ int unsorted_flag, tile_total;
+    const int64_t vs = blockIdx.x;
     const int lane = lane_id();
-    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);
-    if (lane < 16) vrows[vs * 16 + lane] = h.row;
-    int64_t tiles = 0;
+    const bool first = wave_in_block() == 0;
+    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);   // the same in every wave
+    if (first && lane < 16) vrows[vs * 16 + lane] = h.row;
+    int tiles = 0;
     bool take = false;
-    if (h.span > 0 && h.span <= STRIP_BM_WORDS * 32 && h.entries >= min_fill) {
-        const bool sorted = gathered_mark(col, h, bm);
+    if (h.span > 0 && h.span <= STRIP_BM_WORDS * 32 && h.entries >= min_fill) {   // workgroup-uniform
+        const bool sorted = gathered_mark(col, h, bm, &unsorted_flag);
+        if (threadIdx.x == 0) tile_total = 0;
+        __syncthreads();
         const int words = (h.span + 31) >> 5;
         int t = 0;
-        for (int w = lane; w < words; w += WAVE) t += __builtin_popcount(bm[w]);
-        tiles = wave_sum_i32(t);
+        for (int w = (int)threadIdx.x; w < words; w += GATHERED_BLOCK) t += __builtin_popcount(bm[w]);
+        t = wave_sum_i32(t);
+        if (lane == 0 && t) atomicAdd(&tile_total, t);
+        __syncthreads();
+        tiles = tile_total;
         take = sorted && tiles > 0 && h.entries >= (int64_t)min_fill * tiles;
     }
-    if (take && h.row >= 0) owner[h.row] = 3;
-    if (lane == 0) {
-        vstrip_ntiles[vs] = take ? (unsigned int)tiles : 0u;
-        if (take) {
-            spread_add(pc, K_TILES, (unsigned long long)tiles);
-            spread_add(pc, K_NNZ_TILES, (unsigned long long)h.entries);
+    if (first) {
+        if (take && h.row >= 0) owner[h.row] = 3;
+        if (lane == 0) {
+            vstrip_ntiles[vs] = take ? (unsigned int)tiles : 0u;
+            if (take) {
+                spread_add(pc, K_TILES, (unsigned long long)tiles);
+                spread_add(pc, K_NNZ_TILES, (unsigned long long)h.entries);
+            }
         }
     }
 }
 
 // pass 2 of the gathered strips: strip and tile column of every descriptor
-__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_gathered_tiles(
+__global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
     const unsigned long long *__restrict__ sorted_keys,
     int64_t n_cand, int64_t n_vstrips, const unsigned int *__restrict__ vstrip_ntiles,
     const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles) {
-    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
-    const int64_t vs = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
-    if (vs >= n_vstrips) return;
-    if (vstrip_ntiles[vs] == 0) return;
-    unsigned int *bm = bm_all[wave_in_block()];
+    __shared__ unsigned int bm[STRIP_BM_WORDS];
+    __shared__ int unsorted_flag;
+    const int64_t vs = blockIdx.x;
+    if (vstrip_ntiles[vs] == 0) return;              // workgroup-uniform
     const int lane = lane_id();
     const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);
-    (void)gathered_mark(col, h, bm);
+    (void)gathered_mark(col, h, bm, &unsorted_flag);
+    if (wave_in_block() != 0) return;                // the first wave writes the descriptors in column order
     const int words = (h.span + 31) >> 5;
     int64_t run = vstrip_off[vs];
     for (int wb = 0; wb < words; wb += WAVE) {

@@ -526,8 +526,7 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
         ALLOC_TRY(c, c->d_vrows, (size_t)c->n_vstrips * 16 * sizeof(int32_t));
         c->vstrips_cap = c->n_vstrips;
     }
-    const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-    hipLaunchKernelGGL(k_gathered_count, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr, c->d_col,
+    hipLaunchKernelGGL(k_gathered_count, dim3((unsigned)c->n_vstrips), dim3(GATHERED_BLOCK), 0, c->stream, c->d_rowptr, c->d_col,
                        (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
                        c->d_vrows, c->d_owner, c->d_pc);
     HIP_TRY(c, hipGetLastError());
@@ -557,8 +556,7 @@ int plan_tiles_fill(sddmm_ctx *c) {
         HIP_TRY(c, hipGetLastError());
     }
     if (c->n_tiles > c->n_tiles_natural) {
-        const unsigned grid = (unsigned)((c->n_vstrips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-        hipLaunchKernelGGL(k_gathered_tiles, dim3(grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+        hipLaunchKernelGGL(k_gathered_tiles, dim3((unsigned)c->n_vstrips), dim3(GATHERED_BLOCK), 0, c->stream, c->d_rowptr,
                            c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
                            c->d_vstrip_off, c->d_tiles + c->n_tiles_natural);
         HIP_TRY(c, hipGetLastError());
