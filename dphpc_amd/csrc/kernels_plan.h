@@ -15,7 +15,8 @@ struct PlanCounters {
     unsigned long long rows_short, rows_medium, rows_long;
     unsigned long long nnz_short, nnz_medium, nnz_long;
     unsigned long long n_items;    // work items of the wave-per-segment kernel
-    unsigned long long n_tiles, nnz_tiles, tiles_scanned;     // dense-tile path
+    unsigned long long n_tiles, nnz_tiles, tiles_scanned;     // dense-tile path: 16-row and gathered strips
+    unsigned long long n_utiles, nnz_utiles, utiles_scanned;  // dense-tile path: union strips
     unsigned long long n_panels, nnz_panels, panel_items;     // row-panel path
 };
 
@@ -27,13 +28,14 @@ constexpr int SPREAD = 64;
 enum CounterKind {
     K_ROWS_NONEMPTY = 0,
     K_ROWS_SHORT, K_ROWS_MEDIUM, K_ROWS_LONG, K_NNZ_SHORT, K_NNZ_MEDIUM, K_NNZ_LONG,   // row classifier
-    K_TILES, K_NNZ_TILES, K_PANELS, K_NNZ_PANELS,                                      // ownership classifiers
+    K_TILES, K_NNZ_TILES, K_UTILES, K_NNZ_UTILES, K_PANELS, K_NNZ_PANELS,              // ownership classifiers
     K_KINDS
 };
 struct DevCounters {
     unsigned int bad_pattern, coo_unsorted, pad0, pad1;
     unsigned long long n_items, tiles_scanned, panel_items;          // scan totals, one writer each
     unsigned long long n_candidates;                                 // rows offered to the gathered strips
+    unsigned long long utiles_scanned, pad3;                         // scan total of the union strips
     unsigned int max_len[SPREAD];
     unsigned long long k[K_KINDS][SPREAD];
 };
@@ -55,6 +57,7 @@ inline PlanCounters summarize(const DevCounters &d) {
     p.rows_short = sum[K_ROWS_SHORT]; p.rows_medium = sum[K_ROWS_MEDIUM]; p.rows_long = sum[K_ROWS_LONG];
     p.nnz_short = sum[K_NNZ_SHORT]; p.nnz_medium = sum[K_NNZ_MEDIUM]; p.nnz_long = sum[K_NNZ_LONG];
     p.n_tiles = sum[K_TILES]; p.nnz_tiles = sum[K_NNZ_TILES];
+    p.n_utiles = sum[K_UTILES]; p.nnz_utiles = sum[K_NNZ_UTILES]; p.utiles_scanned = d.utiles_scanned;
     p.n_panels = sum[K_PANELS]; p.nnz_panels = sum[K_NNZ_PANELS];
     p.n_items = d.n_items; p.tiles_scanned = d.tiles_scanned; p.panel_items = d.panel_items;
     return p;

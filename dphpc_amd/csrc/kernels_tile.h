@@ -118,6 +118,17 @@ __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, c
     return sorted;
 }
 
+// Every tile lists its 16 B rows (tile_cols, 16 per descriptor, ascending; INT32_MAX
+// where a union tile has fewer): consecutive columns for the aligned tiles.
+__device__ __forceinline__ void write_aligned_cols(int32_t *__restrict__ tile_cols, int64_t at, int tj) {
+    int4 *dst = reinterpret_cast<int4 *>(tile_cols + at * 16);
+    const int c0 = tj * 16;
+    dst[0] = make_int4(c0, c0 + 1, c0 + 2, c0 + 3);
+    dst[1] = make_int4(c0 + 4, c0 + 5, c0 + 6, c0 + 7);
+    dst[2] = make_int4(c0 + 8, c0 + 9, c0 + 10, c0 + 11);
+    dst[3] = make_int4(c0 + 12, c0 + 13, c0 + 14, c0 + 15);
+}
+
 // ---- parallel strip classifier ---------------------------------------------------
 // One wavefront per strip, four strips per workgroup.  The strip's entries are
 // contiguous in the CSR arrays, so the wave streams them 64 per load, several
@@ -153,9 +164,10 @@ __device__ __forceinline__ void wave_lds_order() {
 
 // Streams entries [e0, e1).  Returns the number of tile-column changes, or -1 as
 // soon as it exceeds `budget`; *descents receives the number of entries whose
-// column does not exceed the column stored before them.  SET_BITS: also sets bit
-// (col>>4) - lo in bm after every change.
-template <bool SET_BITS>
+// column does not exceed the column stored before them.  BITS == 1: also sets bit
+// (col>>4) - lo in bm after every change (tile columns); BITS == 2: sets bit col - lo
+// for every entry (columns).
+template <int BITS>
 __device__ __forceinline__ int64_t strip_scan(const int32_t *__restrict__ col, int e0, int e1, int64_t budget,
                                               int lo, int span, unsigned int *bm, int64_t *descents) {
     const int lane = lane_id();
@@ -183,9 +195,12 @@ __device__ __forceinline__ int64_t strip_scan(const int32_t *__restrict__ col, i
             const int prev = __builtin_amdgcn_update_dpp(carry, cur[u], 0x138, 0xF, 0xF, false);
             carry = __builtin_amdgcn_readlane(cur[u], WAVE - 1);
             const bool change = valid && (cur[u] >> 4) != (prev >> 4);
-            if constexpr (SET_BITS) {
+            if constexpr (BITS == 1) {
                 const int t = (cur[u] >> 4) - lo;
                 if (change && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
+            } else if constexpr (BITS == 2) {
+                const int t = cur[u] - lo;
+                if (valid && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
             }
             changes += __popcll(__ballot(change));
             desc += __popcll(__ballot(valid && cur[u] <= prev));
@@ -199,10 +214,12 @@ __device__ __forceinline__ int64_t strip_scan(const int32_t *__restrict__ col, i
 }
 
 // From the first and last entry of each of the 16 rows (lane i < 16: row i, whose
-// rowptr is lane_rp): the strip's column span in tile columns, [lo, lo + span)
+// rowptr is lane_rp): the strip's column span in tile columns (SHIFT 4) or columns
+// (SHIFT 0), [lo, lo + span)
 // (exact when the rows are sorted; span <= 0 when they are not or no row has an
 // entry), and the number of row starts whose column does not exceed the column
 // stored before them -- the descents a sorted strip is allowed.
+template <int SHIFT = 4>
 __device__ __forceinline__ void strip_bounds(const int32_t *__restrict__ col, int lane_rp, int e0, int *lo, int *span,
                                              int *boundary_descents) {
     const int lane = lane_id();
@@ -211,8 +228,8 @@ __device__ __forceinline__ void strip_bounds(const int32_t *__restrict__ col, in
     const int first_col = has ? col[lane_rp] : INT32_MAX;
     const int last_col = has ? col[nxt - 1] : -1;
     const int before = has && lane_rp > e0 ? col[lane_rp - 1] : -1;
-    const int l = __builtin_amdgcn_readfirstlane(min16(has ? first_col >> 4 : INT32_MAX));
-    const int hneg = __builtin_amdgcn_readfirstlane(min16(has ? -(last_col >> 4) : 1));
+    const int l = __builtin_amdgcn_readfirstlane(min16(has ? first_col >> SHIFT : INT32_MAX));
+    const int hneg = __builtin_amdgcn_readfirstlane(min16(has ? -(last_col >> SHIFT) : 1));
     *lo = l;
     *span = l == INT32_MAX ? 0 : -hneg - l + 1;
     *boundary_descents = __popcll(__ballot(has && first_col <= before));
@@ -246,13 +263,13 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
     // before anything else is read
     constexpr int FIRST = WAVE * STRIP_UNROLL;
     if (max_tiles > 0 &&
-        strip_scan<false>(col, e0, e1 - e0 > FIRST ? e0 + FIRST : e1, budget, 0, 0, nullptr, &descents) >= 0) {
+        strip_scan<0>(col, e0, e1 - e0 > FIRST ? e0 + FIRST : e1, budget, 0, 0, nullptr, &descents) >= 0) {
         int lo, span, allowed;
         strip_bounds(col, lane_rp, e0, &lo, &span, &allowed);
         if (span > STRIP_BM_WORDS * 32) {
             // too wide for the bitmap: scan without it, then merge the 16 rows in the first
             // 16 lanes if the strip is still a candidate
-            const int64_t ch = strip_scan<false>(col, e0, e1, budget, 0, 0, nullptr, &descents);
+            const int64_t ch = strip_scan<0>(col, e0, e1, budget, 0, 0, nullptr, &descents);
             if (ch >= 0 && descents == allowed) {
                 int t = 0;
                 if (lane < 16) {
@@ -267,7 +284,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
             const int words = (span + 31) >> 5;
             for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
             wave_lds_order();
-            const int64_t ch = strip_scan<true>(col, e0, e1, budget, lo, span, bm, &descents);
+            const int64_t ch = strip_scan<1>(col, e0, e1, budget, lo, span, bm, &descents);
             wave_lds_order();
             if (ch >= 0 && descents == allowed) {
                 int t = 0;
@@ -294,7 +311,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
 __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips,
     const unsigned int *__restrict__ strip_ntiles, const unsigned int *__restrict__ strip_off,
-    TileDesc *__restrict__ tiles) {
+    TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols) {
     __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][STRIP_BM_WORDS];
     const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
     if (strip >= n_strips) return;
@@ -315,6 +332,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
                 d->off[lane] = first;
                 d->mask[lane] = (uint16_t)mask;
                 if (lane == 0) { d->strip = (int32_t)strip; d->tj = tj; d->pad[0] = 1; d->pad[1] = 0; }
+                tile_cols[at * 16 + lane] = tj * 16 + lane;
                 ++at;
                 return true;
             });
@@ -325,7 +343,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
     for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
     wave_lds_order();
     int64_t descents;
-    (void)strip_scan<true>(col, e0, e1, INT64_MAX, lo, span, bm, &descents);
+    (void)strip_scan<1>(col, e0, e1, INT64_MAX, lo, span, bm, &descents);
     wave_lds_order();
     int64_t run = first_desc;
     for (int wb = 0; wb < words; wb += WAVE) {
@@ -342,10 +360,123 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_tiles(
             const int b = __builtin_ctz(x);
             x &= x - 1;
             *reinterpret_cast<int4 *>(tiles + at) = make_int4((int)strip, lo + w * 32 + b, 0, 0);
+            write_aligned_cols(tile_cols, at, lo + w * 32 + b);
             ++at;
         }
         run += __builtin_amdgcn_readlane(incl, WAVE - 1);
     }
+}
+
+// ---- union strips --------------------------------------------------------------------
+// A 16-row strip whose rows are similar but not aligned to 16-column blocks (mesh
+// rows that share most of their neighbours) wastes the aligned tiles: its columns are
+// spread over many of them.  Here the strip's tiles are cut from the sorted UNION of
+// its column lists instead, 16 union columns per tile, so a B row is gathered once
+// for the rows of the strip that have it -- the role of the active-column lists of
+// src/competitors/gpu/gpu_preprocessing.hpp:57-141.  Same machinery as above with a
+// bitmap of columns instead of tile columns: popcount = size of the union, the rank
+// of a column gives its tile and its position in the tile.
+constexpr int UNION_BM_WORDS = 4096;          // a column span of 131072 per strip
+
+__device__ __forceinline__ int max16(int v) { return -min16(-v); }
+
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_union_count(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips, int min_fill,
+    unsigned char *__restrict__ owner, unsigned int *__restrict__ ustrip_ntiles, DevCounters *pc) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][UNION_BM_WORDS];
+    const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
+    if (strip >= n_strips) return;
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const int64_t r = strip * 16 + lane;
+    const int lane_rp = rowptr[r < M ? r : M];
+    const int e0 = __builtin_amdgcn_readlane(lane_rp, 0), e1 = __builtin_amdgcn_readlane(lane_rp, 16);
+    const int64_t entries = (int64_t)e1 - (int64_t)e0;
+    // the strip must be free as a whole, and even its longest row alone must not need
+    // more tiles than the threshold allows
+    const bool owned = lane < 16 && r < M && owner[r] != 0;
+    const int next_rp = __shfl_down(lane_rp, 1, WAVE);          // every lane takes part in the permute
+    const int len = lane < 16 ? next_rp - lane_rp : 0;
+    const int longest = __builtin_amdgcn_readfirstlane(max16(lane < 16 ? len : 0));
+    int64_t tiles = 0;
+    bool take = false;
+    if (__ballot(owned) == 0ull && entries >= (int64_t)min_fill * ((longest + 15) / 16) && entries >= min_fill) {
+        int lo, span, allowed;
+        strip_bounds<0>(col, lane_rp, e0, &lo, &span, &allowed);
+        if (span > 0 && span <= UNION_BM_WORDS * 32) {
+            const int words = (span + 31) >> 5;
+            for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
+            wave_lds_order();
+            int64_t descents = 0;
+            (void)strip_scan<2>(col, e0, e1, INT64_MAX, lo, span, bm, &descents);
+            wave_lds_order();
+            if (descents == allowed) {
+                int t = 0;
+                for (int w = lane; w < words; w += WAVE) t += __builtin_popcount(bm[w]);
+                tiles = (wave_sum_i32(t) + 15) / 16;
+                take = tiles > 0 && entries >= (int64_t)min_fill * tiles;
+            }
+        }
+    }
+    if (take && lane < 16 && r < M) owner[r] = 4;
+    if (lane == 0) {
+        ustrip_ntiles[strip] = take ? (unsigned int)tiles : 0u;
+        if (take) {
+            spread_add(pc, K_UTILES, (unsigned long long)tiles);
+            spread_add(pc, K_NNZ_UTILES, (unsigned long long)entries);
+        }
+    }
+}
+
+// descriptors of the union strips: header and the 16 union columns of every tile
+__global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_union_tiles(
+    const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M, int64_t n_strips,
+    const unsigned int *__restrict__ ustrip_ntiles, const unsigned int *__restrict__ ustrip_off,
+    TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols) {
+    __shared__ unsigned int bm_all[STRIPS_PER_BLOCK][UNION_BM_WORDS];
+    const int64_t strip = (int64_t)blockIdx.x * STRIPS_PER_BLOCK + wave_in_block();
+    if (strip >= n_strips) return;
+    const unsigned int ntiles = ustrip_ntiles[strip];
+    if (ntiles == 0) return;
+    unsigned int *bm = bm_all[wave_in_block()];
+    const int lane = lane_id();
+    const int64_t r = strip * 16 + lane;
+    const int lane_rp = rowptr[r < M ? r : M];
+    const int e0 = __builtin_amdgcn_readlane(lane_rp, 0), e1 = __builtin_amdgcn_readlane(lane_rp, 16);
+    int lo, span, allowed;
+    strip_bounds<0>(col, lane_rp, e0, &lo, &span, &allowed);
+    const int words = (span + 31) >> 5;
+    for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
+    wave_lds_order();
+    int64_t descents = 0;
+    (void)strip_scan<2>(col, e0, e1, INT64_MAX, lo, span, bm, &descents);
+    wave_lds_order();
+    const int64_t first = ustrip_off[strip];
+    int64_t run = 0;                              // union columns before this batch of words
+    for (int wb = 0; wb < words; wb += WAVE) {
+        const int w = wb + lane;
+        unsigned int x = w < words ? bm[w] : 0u;
+        const int n = __builtin_popcount(x);
+        int incl = n;
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const int up = __shfl_up(incl, o, WAVE);
+            if (lane >= o) incl += up;
+        }
+        int64_t rank = run + (incl - n);
+        while (x) {
+            const int b = __builtin_ctz(x);
+            x &= x - 1;
+            const int c = lo + w * 32 + b;
+            const int64_t t = first + (rank >> 4);
+            tile_cols[t * 16 + (rank & 15)] = c;
+            if ((rank & 15) == 0) *reinterpret_cast<int4 *>(tiles + t) = make_int4((int)strip, c >> 4, 0, 0);
+            ++rank;
+        }
+        run += __builtin_amdgcn_readlane(incl, WAVE - 1);
+    }
+    // the last tile of the strip may hold fewer than 16 columns
+    const int tail = (int)(run & 15);
+    if (tail != 0 && lane >= tail && lane < 16) tile_cols[(first + ntiles - 1) * 16 + lane] = INT32_MAX;
 }
 
 // ---- gathered strips ---------------------------------------------------------------
@@ -434,7 +565,7 @@ __device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, c
     const int si = __builtin_amdgcn_readlane(h.s, wi), ei = __builtin_amdgcn_readlane(h.e, wi);
     if (ei > si) {                                   // wave-uniform
         int64_t descents = 0;
-        (void)strip_scan<true>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
+        (void)strip_scan<1>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
         if (descents != 0 && lane_id() == 0) atomicOr(unsorted_flag, 1);
     }
     __syncthreads();
@@ -487,7 +618,7 @@ __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
     const unsigned long long *__restrict__ sorted_keys,
     int64_t n_cand, int64_t n_vstrips, const unsigned int *__restrict__ vstrip_ntiles,
-    const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles) {
+    const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols) {
     __shared__ unsigned int bm[STRIP_BM_WORDS];
     __shared__ int unsorted_flag;
     const int64_t vs = blockIdx.x;
@@ -512,6 +643,7 @@ __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
             const int b = __builtin_ctz(x);
             x &= x - 1;
             *reinterpret_cast<int4 *>(tiles + at) = make_int4(GATHERED_BASE + (int)vs, h.lo + w * 32 + b, 0, 0);
+            write_aligned_cols(tile_cols, at, h.lo + w * 32 + b);
             ++at;
         }
         run += __builtin_amdgcn_readlane(incl, WAVE - 1);
@@ -520,9 +652,12 @@ __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
 
 // pass 3: one thread per (descriptor, row): CSR position of the row's first entry
 // at or after the tile's first column, and the mask of the tile's columns present.
+// Bit n of the mask stands for the n-th of the tile's 16 columns; a row's entries
+// inside a tile are consecutive in CSR, in the order of the tile's columns.
 __global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ rowptr,
                                                    const int32_t *__restrict__ col, int M,
                                                    const int32_t *__restrict__ vrows,
+                                                   const int32_t *__restrict__ tile_cols,
                                                    TileDesc *__restrict__ tiles, int64_t n_tiles) {
     const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t t = slot >> 4;
@@ -531,12 +666,23 @@ __global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ r
     TileDesc *d = tiles + t;
     const int4 head = *reinterpret_cast<const int4 *>(d);     // strip, tj, pad[0], pad[1]
     if (head.z != 0) return;                                   // written by the merging walk
-    const int tj = head.y;
     const int64_t row = head.x >= GATHERED_BASE ? (int64_t)vrows[(int64_t)(head.x - GATHERED_BASE) * 16 + sub]
                                                 : (int64_t)head.x * 16 + sub;
     int p = 0, end = 0;
     if (row >= 0 && row < M) { p = rowptr[row]; end = rowptr[row + 1]; }
-    const int target = tj * 16;
+    int tc[16];
+    {
+        const int4 *src = reinterpret_cast<const int4 *>(tile_cols + t * 16);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int4 v = src[k];
+            tc[4 * k] = v.x; tc[4 * k + 1] = v.y; tc[4 * k + 2] = v.z; tc[4 * k + 3] = v.w;
+        }
+    }
+    int top = tc[0];                                           // last real column of the tile
+#pragma unroll
+    for (int k = 1; k < 16; ++k) top = tc[k] != INT32_MAX ? tc[k] : top;
+    const int target = tc[0];
     int a = p, b = end;
     while (a < b) {
         const int mid = a + ((b - a) >> 1);
@@ -549,8 +695,14 @@ __global__ __launch_bounds__(256) void k_tile_rows(const int32_t *__restrict__ r
 #pragma unroll
         for (int j = 0; j < 16; ++j) cs[j] = col[a + j < last ? a + j : last];
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            if (a + j <= last && (cs[j] >> 4) == tj) mask |= 1u << (cs[j] & 15);
+        for (int j = 0; j < 16; ++j) {
+            if (a + j <= last && cs[j] <= top) {
+                int n = 0;                                     // number of tile columns below this one
+#pragma unroll
+                for (int k = 0; k < 16; ++k) n += tc[k] < cs[j] ? 1 : 0;
+                mask |= 1u << n;
+            }
+        }
     }
     d->off[sub] = a;
     d->mask[sub] = (uint16_t)mask;
@@ -607,9 +759,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 // tiles [w*tiles_per_wave, (w+1)*tiles_per_wave) on the calling wavefront
 template <int DT, int STEPS>
 __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
-                                          const int32_t *__restrict__ vrows, const TileDesc *__restrict__ tiles,
-                                          int64_t n_tiles, int tiles_per_wave, const float *__restrict__ sval,
-                                          float *__restrict__ P, int64_t w) {
+                                          const int32_t *__restrict__ vrows, const int32_t *__restrict__ tile_cols,
+                                          const TileDesc *__restrict__ tiles, int64_t n_tiles, int tiles_per_wave,
+                                          const float *__restrict__ sval, float *__restrict__ P, int64_t w) {
     int64_t t = w * tiles_per_wave;
     if (t >= n_tiles) return;
     int64_t t_end = t + tiles_per_wave;
@@ -633,7 +785,7 @@ __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void
     };
 
     struct Desc {
-        int strip, tj;
+        int strip, bcol;    // bcol: the B row this lane loads (memory layout)
         int4 off;
         uint2 mask;
     };
@@ -648,15 +800,15 @@ __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void
         const TileDesc *d = tiles + ti;
         Desc r;
         r.strip = d->strip;
-        r.tj = d->tj;
+        r.bcol = tile_cols[ti * 16 + lrow];
         r.off = *(const int4 *)&d->off[q * 4];
         r.mask = *(const uint2 *)&d->mask[q * 4];
         return r;
     };
     auto load_oper = [&](const Desc &d) {
         Oper o;
-        int64_t brow = (int64_t)d.tj * 16 + lrow;
-        brow = brow < N ? brow : N - 1;   // columns past N are never in a mask
+        int64_t brow = d.bcol;
+        brow = brow < N ? brow : N - 1;   // columns past N (and the filler of a short union tile) are never in a mask
         const uint4 *src = Bu + brow * ROW_UNITS + lunit;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
@@ -726,12 +878,13 @@ __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void
 template <int DT, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
                                                 const int32_t *__restrict__ vrows,
+                                                const int32_t *__restrict__ tile_cols,
                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                 int tiles_per_wave, const float *__restrict__ sval,
                                                 float *__restrict__ P, int64_t nblocks) {
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
-    tile_wave<DT, STEPS>(A, B, M, N, vrows, tiles, n_tiles, tiles_per_wave, sval, P,
+    tile_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, tiles_per_wave, sval, P,
                          blk * WAVES_PER_BLOCK + wave_in_block());
 }
 
@@ -749,13 +902,14 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
                                                       int N, int ts, int rpw, int64_t short_blocks,
                                                       const RowItem *__restrict__ items, int64_t n_items,
                                                       const int32_t *__restrict__ vrows,
+                                                      const int32_t *__restrict__ tile_cols,
                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                       int tiles_per_wave, int64_t tile_blocks, int64_t nblocks) {
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int64_t tiles_before = blk * tile_blocks / nblocks;
     if (((blk + 1) * tile_blocks / nblocks) != tiles_before) {
-        tile_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tiles, n_tiles, tiles_per_wave, sval, P,
+        tile_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, tiles_per_wave, sval, P,
                                    tiles_before * WAVES_PER_BLOCK + wave_in_block());
         return;
     }

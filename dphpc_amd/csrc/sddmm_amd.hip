@@ -70,7 +70,12 @@ struct sddmm_ctx {
     int64_t n_tiles = 0, tiles_cap = 0, nnz_tiles = 0;
     int tile_steps = 0, tiles_per_wave = 8;
     bool tiles_active = false;       // d_tiles describes the current pattern
-    int64_t n_tiles_natural = 0;     // descriptors of 16-row strips come first, gathered strips after
+    int64_t n_tiles_natural = 0;     // descriptors: 16-row strips first, then union strips, then gathered strips
+    int64_t n_tiles_union = 0, nnz_tiles_union = 0;
+    unsigned int *d_ustrip_ntiles = nullptr, *d_ustrip_off = nullptr;
+    int64_t ustrips_cap = 0;
+    int32_t *d_tile_cols = nullptr;  // 16 B rows per descriptor
+    bool union_counted = false;
     // gathered strips: candidate rows, sorted by first column, 16 per strip
     unsigned long long *d_cand_keys = nullptr, *d_sorted_keys = nullptr;   // (first column << 32) | row
     int32_t *d_vrows = nullptr;
@@ -153,6 +158,9 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_strip_ntiles);
     dfree(c->d_strip_off);
     dfree(c->d_tiles);
+    dfree(c->d_tile_cols);
+    dfree(c->d_ustrip_ntiles); dfree(c->d_ustrip_off);
+    c->ustrips_cap = 0;
     dfree(c->d_cand_keys); dfree(c->d_sorted_keys);
     dfree(c->d_vrows); dfree(c->d_sort_tmp); dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off);
     c->sort_tmp_bytes = 0;
@@ -342,8 +350,8 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
                                (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
                                (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
                                c->dP, c->sM, c->N, c->ts, c->rpw, short_blocks, c->d_items, c->n_items,
-                               (const int32_t *)c->d_vrows, (const TileDesc *)c->d_tiles, c->n_tiles,
-                               c->tiles_per_wave, tile_blocks, nblocks);
+                               (const int32_t *)c->d_vrows, (const int32_t *)c->d_tile_cols,
+                               (const TileDesc *)c->d_tiles, c->n_tiles, c->tiles_per_wave, tile_blocks, nblocks);
             launched = true;
         }
     });
@@ -432,11 +440,12 @@ int begin_ownership(sddmm_ctx *c) {
     HIP_TRY(c, hipMemsetAsync(c->d_owner, 0, (size_t)bytes, c->stream));
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_TILES][0], 0,
                               sizeof(unsigned long long) * SPREAD * (K_NNZ_PANELS - K_TILES + 1), c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 3 * sizeof(unsigned long long), c->stream));
+    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 5 * sizeof(unsigned long long), c->stream));
     c->owner_active = true;
     c->tiles_active = false;
-    c->n_tiles = c->nnz_tiles = c->n_tiles_natural = 0;
+    c->n_tiles = c->nnz_tiles = c->n_tiles_natural = c->n_tiles_union = c->nnz_tiles_union = 0;
     c->n_cand = c->n_vstrips = 0;
+    c->union_counted = false;
     c->n_panel_items = c->n_panels = c->nnz_panels = 0;
     return SDDMM_OK;
 }
@@ -480,7 +489,33 @@ int take_tile_counts(sddmm_ctx *c) {
     c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
     if (c->tile_steps != 0 && (int64_t)c->pc.tiles_scanned != c->n_tiles)
         return fail(c, SDDMM_ERR_HIP, "internal: tile scan disagrees with tile count");
+    c->n_tiles_union = c->union_counted ? (int64_t)c->pc.n_utiles : 0;
+    c->nnz_tiles_union = c->union_counted ? (int64_t)c->pc.nnz_utiles : 0;
+    if (c->union_counted && (int64_t)c->pc.utiles_scanned != c->n_tiles_union)
+        return fail(c, SDDMM_ERR_HIP, "internal: union tile scan disagrees with tile count");
+    c->n_tiles += c->n_tiles_union;
+    c->nnz_tiles += c->nnz_tiles_union;
     return SDDMM_OK;
+}
+
+// Union strips among the 16-row strips nobody owns yet (launch only; after the panel
+// detector, before the candidates of the gathered strips).
+int plan_union_count(sddmm_ctx *c, int min_fill) {
+    if (c->tile_steps == 0) return SDDMM_OK;
+    const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
+    if (n_strips > c->ustrips_cap) {
+        dfree(c->d_ustrip_ntiles);
+        dfree(c->d_ustrip_off);
+        ALLOC_TRY(c, c->d_ustrip_ntiles, (size_t)n_strips * sizeof(unsigned int));
+        ALLOC_TRY(c, c->d_ustrip_off, (size_t)n_strips * sizeof(unsigned int));
+        c->ustrips_cap = n_strips;
+    }
+    const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+    hipLaunchKernelGGL(k_union_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                       c->d_col, c->sM, n_strips, min_fill, c->d_owner, c->d_ustrip_ntiles, c->d_pc);
+    HIP_TRY(c, hipGetLastError());
+    c->union_counted = true;
+    return device_scan(c, c->d_ustrip_ntiles, c->d_ustrip_off, n_strips, &c->d_pc->utiles_scanned);
 }
 
 // Candidates of the gathered strips (launch only; the count arrives with the next
@@ -534,9 +569,9 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
     if (rc) return rc;
     rc = fetch_counters(c);
     if (rc) return rc;
-    c->n_tiles = (int64_t)c->pc.n_tiles;
-    c->nnz_tiles = (int64_t)c->pc.nnz_tiles;
-    if ((int64_t)c->pc.tiles_scanned != c->n_tiles - c->n_tiles_natural)
+    c->n_tiles = (int64_t)c->pc.n_tiles + c->n_tiles_union;
+    c->nnz_tiles = (int64_t)c->pc.nnz_tiles + c->nnz_tiles_union;
+    if ((int64_t)c->pc.tiles_scanned != (int64_t)c->pc.n_tiles - c->n_tiles_natural)
         return fail(c, SDDMM_ERR_HIP, "internal: gathered tile scan disagrees with tile count");
     return SDDMM_OK;
 }
@@ -545,24 +580,37 @@ int plan_tiles_fill(sddmm_ctx *c) {
     if (c->n_tiles == 0) return SDDMM_OK;
     if (c->n_tiles > c->tiles_cap) {
         dfree(c->d_tiles);
+        dfree(c->d_tile_cols);
+        c->tiles_cap = 0;
         ALLOC_TRY(c, c->d_tiles, (size_t)c->n_tiles * sizeof(TileDesc));
+        ALLOC_TRY(c, c->d_tile_cols, (size_t)c->n_tiles * 16 * sizeof(int32_t));
         c->tiles_cap = c->n_tiles;
     }
     if (c->n_tiles_natural > 0) {
         const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
         const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
         hipLaunchKernelGGL(k_strip_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
-                           c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles);
+                           c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles, c->d_tile_cols);
         HIP_TRY(c, hipGetLastError());
     }
-    if (c->n_tiles > c->n_tiles_natural) {
+    if (c->n_tiles_union > 0) {
+        const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
+        const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
+        hipLaunchKernelGGL(k_union_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+                           c->d_col, c->sM, n_strips, c->d_ustrip_ntiles, c->d_ustrip_off,
+                           c->d_tiles + c->n_tiles_natural, c->d_tile_cols + c->n_tiles_natural * 16);
+        HIP_TRY(c, hipGetLastError());
+    }
+    if (c->n_tiles > c->n_tiles_natural + c->n_tiles_union) {
         hipLaunchKernelGGL(k_gathered_tiles, dim3((unsigned)c->n_vstrips), dim3(GATHERED_BLOCK), 0, c->stream, c->d_rowptr,
                            c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
-                           c->d_vstrip_off, c->d_tiles + c->n_tiles_natural);
+                           c->d_vstrip_off, c->d_tiles + c->n_tiles_natural + c->n_tiles_union,
+                           c->d_tile_cols + (c->n_tiles_natural + c->n_tiles_union) * 16);
         HIP_TRY(c, hipGetLastError());
     }
     hipLaunchKernelGGL(k_tile_rows, dim3((unsigned)((c->n_tiles * 16 + 255) / 256)), dim3(256), 0, c->stream,
-                       c->d_rowptr, c->d_col, c->sM, (const int32_t *)c->d_vrows, c->d_tiles, c->n_tiles);
+                       c->d_rowptr, c->d_col, c->sM, (const int32_t *)c->d_vrows, (const int32_t *)c->d_tile_cols,
+                       c->d_tiles, c->n_tiles);
     HIP_TRY(c, hipGetLastError());
     c->tiles_active = true;
     c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 4));
@@ -678,7 +726,7 @@ void launch_tile_t(sddmm_ctx *c) {
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     hipLaunchKernelGGL((k_tile<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
-                       (const TileDesc *)c->d_tiles, c->n_tiles,
+                       (const int32_t *)c->d_tile_cols, (const TileDesc *)c->d_tiles, c->n_tiles,
                        c->tiles_per_wave, (const float *)c->d_sval, c->dP, nblocks);
 }
 template <int DT>
@@ -818,6 +866,10 @@ int do_plan(sddmm_ctx *c, int strategy) {
                 if (rc) return rc;
             } else {
                 c->panels_flagged = false;
+            }
+            if (resolved == SDDMM_AUTO && env_int("SDDMM_UNION", 1) != 0) {
+                rc = plan_union_count(c, std::max(1, env_int("SDDMM_UNION_FILL", tile_fill)));
+                if (rc) return rc;
             }
             if (gathered) {
                 rc = plan_gathered_candidates(c, std::max(16, env_int("SDDMM_GATHERED_MIN", 64)));

@@ -71,7 +71,11 @@ enum sddmm_strategy {
                              src/competitors/gpu/gpu_shared.cu:18-88 and
                              gpu_preprocessing.cu:18-96: B reused across a row panel) */
     SDDMM_MFMA_TILE = 5,  /* near-dense 16x16 tiles on MFMA, remainder on AUTO's
-                             gather kernels (the role of gpu_tensor.cu:27-99)         */
+                             gather kernels (the role of gpu_tensor.cu:27-99).  AUTO
+                             also cuts tiles from the union of the columns of 16
+                             similar rows (the active-column lists of
+                             gpu_preprocessing.hpp:57-141) and from near-dense rows
+                             gathered by column window                                */
     SDDMM_EXACT = 6       /* one lane per entry, k ascending, separate fp32 multiply
                              and add: bit-identical to cpu_basic.hpp:18-51            */
 };

@@ -645,3 +645,78 @@ def test_gathered_strips(engine_factory, monkeypatch, K, dtype):
     off, st3 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
     assert st3.mfma_tiles == 0
     assert_parity(off, rowptr, col, val, A, B, what="gathered strips off")
+
+
+def _host_union_model(M, rowptr, col, min_fill, span_limit=131072):
+    """Union strips as the device must find them when no other path owns a row: a
+    16-row strip is taken iff its rows are strictly increasing, its column span fits
+    the classifier and it holds at least min_fill entries per tile of 16 union columns."""
+    tiles = entries = 0
+    for s in range((M + 15) // 16):
+        lo, hi = rowptr[s * 16], rowptr[min(M, s * 16 + 16)]
+        if hi - lo < min_fill:
+            continue
+        rows = [col[rowptr[r]:rowptr[r + 1]].astype(np.int64) for r in range(s * 16, min(M, s * 16 + 16))]
+        if any(len(c) > 1 and (np.diff(c) <= 0).any() for c in rows):
+            continue
+        u = np.unique(np.concatenate(rows))
+        if u[-1] - u[0] + 1 > span_limit:
+            continue
+        t = (len(u) + 15) // 16
+        if hi - lo >= min_fill * t:
+            tiles += t
+            entries += hi - lo
+    return tiles, entries
+
+
+@pytest.mark.parametrize("K,dtype", [(32, "f32"), (128, "f32"), (64, "bf16")])
+def test_union_strips(engine_factory, monkeypatch, K, dtype):
+    """Rows that share most of their columns without being identical or aligned to
+    16-column blocks: the tiles are cut from the union of the strip's columns."""
+    monkeypatch.setenv("SDDMM_GATHERED", "0")
+    rng = np.random.default_rng(600 + K)
+    M, N = 16 * 40 + 5, 300_000
+    rows = []
+    for g in range(M // 16 + 1):
+        kind = g % 5
+        if kind == 0:                                    # 16 similar rows, scattered base
+            base = np.sort(rng.choice(60_000, 150, replace=False)) + int(rng.integers(0, N - 60_000))
+            grp = [base[rng.random(150) > 0.15] for _ in range(16)]
+        elif kind == 1:                                  # two different groups of 8 similar rows
+            grp = []
+            for _ in range(2):
+                base = np.sort(rng.choice(5_000, 120, replace=False)) + int(rng.integers(0, N - 5_000))
+                grp += [base[rng.random(120) > 0.1] for _ in range(8)]
+        elif kind == 2:                                  # unrelated rows: the union is as large as the strip
+            grp = [np.sort(rng.choice(100_000, 40, replace=False)) for _ in range(16)]
+        elif kind == 3:                                  # similar rows over a span too wide for the classifier
+            base = np.sort(rng.choice(N, 150, replace=False))
+            grp = [base[rng.random(150) > 0.1] for _ in range(16)]
+        else:                                            # similar rows, one of them not sorted
+            base = np.sort(rng.choice(3_000, 100, replace=False))
+            grp = [base[rng.random(100) > 0.1] for _ in range(16)]
+            grp[3] = np.concatenate([grp[3][:2][::-1], grp[3][2:]])
+        rows += grp
+    rows = rows[:M]
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == "bf16":
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B, ops, dt = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K), (Ab, Bb), capi.BF16
+    else:
+        ops, dt = (A, B), capi.F32
+    fill = 80 if K * (2 if dtype == "bf16" else 4) <= 128 else 56
+    got, st = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert_parity(got, rowptr, col, val, A, B, what="union strips")
+    want = _host_union_model(M, rowptr, col, fill)
+    assert want[0] > 0 and st.panels == 0
+    assert (st.mfma_tiles, st.nnz_mfma) == want
+    assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
+    monkeypatch.setenv("SDDMM_UNION", "0")
+    off, st0 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st0.mfma_tiles == 0
+    assert_parity(off, rowptr, col, val, A, B, what="union strips off")
