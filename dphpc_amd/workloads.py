@@ -223,6 +223,29 @@ def dense_tiles(K=128, M=4562, N=5761, tile_frac=0.09377, seed=SEED_BASE + 5, bf
                     A_bits=Ab.reshape(M, K), B_bits=Bb.reshape(N, K), meta={"tiles": n_tiles})
 
 
+# --------------------------------------------------------------------------- 6
+def similar_rows(K=32, M=40000, group=16, base_len=200, drop=0.10, window=800, seed=SEED_BASE + 6):
+    """Groups of `group` consecutive rows that share most of their columns without being
+    identical (rows of a mesh with mostly common neighbours): every group draws base_len
+    columns inside a window of `window` columns, every row of the group drops a fraction
+    `drop` of them.  Not one of the benchmark configurations of the reference; the shape
+    the union strips are for."""
+    rng = np.random.default_rng(seed)
+    N = M
+    keys = []
+    for g in range(M // group):
+        c0 = int(rng.integers(0, N - window + 1))
+        base = np.sort(rng.choice(window, size=base_len, replace=False)) + c0
+        for i in range(group):
+            keep = base[rng.random(base_len) >= drop]
+            keys.append((g * group + i) * np.int64(N) + keep.astype(np.int64))
+    rowptr, col = _csr_from_keys(M, N, np.concatenate(keys))
+    sval = rng.random(len(col), dtype=np.float32)
+    return Workload("similar_rows", M, N, K, rowptr, col, sval,
+                    _dense(rng, M, K, "uniform"), _dense(rng, N, K, "uniform"),
+                    meta={"group": group, "base_len": base_len, "drop": drop})
+
+
 # ---------------------------------------------------------------------------
 # name -> (generator, kwargs at benchmark size, kwargs at test size)
 CONFIGS = {
@@ -231,6 +254,7 @@ CONFIGS = {
     "power_law": (power_law, {}, dict(M=60000, nnz_target=600000, trunc=4000)),
     "mixed_density": (mixed_density, {}, dict(M=3000, window=700)),
     "dense_tiles": (dense_tiles, {}, dict(M=1140, N=1445)),
+    "similar_rows": (similar_rows, {}, dict(M=1600)),
 }
 
 
