@@ -192,3 +192,86 @@ def test_strip_classifier_matches_host_model(engine_factory, monkeypatch, seed):
     ok, worst, i = O.check_values(e.values(), ref, mag=mag)
     assert ok, (seed, "AUTO with gathered strips", i, worst)
     e.close()
+
+
+def build_similarity_case(seed):
+    """Mixtures aimed at the ownership logic of the tile paths: groups of similar rows
+    (union strips), near-dense rows in windows (gathered strips), identical groups
+    (panels), aligned dense tiles, with short, long, empty, unsorted and duplicated rows
+    in between; K, N and the operand type vary with the seed."""
+    rng = np.random.default_rng(90000 + seed)
+    N = int(rng.choice([300, 5000, 100000, 400000]))
+    K = int(rng.choice([16, 32, 64, 128, 256, 24]))
+    dt = str(rng.choice(["f32", "f32", "bf16", "f16"])) if K % 8 == 0 else "f32"
+    rows = []
+    target = int(rng.integers(30, 700))
+    while len(rows) < target:
+        kind = int(rng.integers(0, 8))
+        if kind == 0:
+            g = int(rng.choice([3, 8, 16, 16, 20, 32]))
+            bl = int(rng.integers(20, min(N, 300)))
+            win = int(min(N, bl * rng.integers(1, 30)))
+            base = np.sort(rng.choice(win, bl, replace=False)) + int(rng.integers(0, N - win + 1))
+            flip = float(rng.choice([0.0, 0.05, 0.3]))
+            rows += [base[rng.random(bl) >= flip] for _ in range(g)]
+        elif kind == 1:
+            win = int(min(N, rng.integers(100, 1500)))
+            c0 = int(rng.integers(0, N - win + 1))
+            rows.append(c0 + np.nonzero(rng.random(win) < rng.choice([0.3, 0.6, 0.95]))[0])
+        elif kind == 2:
+            rows += [np.sort(rng.choice(N, int(rng.integers(0, 15)), replace=False)) for _ in range(int(rng.integers(1, 30)))]
+        elif kind == 3:
+            rows.append(np.sort(rng.choice(N, int(rng.integers(min(N, 100), min(N, 3000))), replace=False)))
+        elif kind == 4:
+            rows += [np.zeros(0, np.int64)] * int(rng.integers(1, 20))
+        elif kind == 5:
+            base = np.sort(rng.choice(N, int(rng.integers(4, min(N, 200))), replace=False))
+            rows += [base.copy() for _ in range(int(rng.choice([8, 16, 24])))]
+        elif kind == 6:
+            tcs = np.sort(rng.choice(max(1, N // 16), int(rng.integers(1, 6)), replace=False))
+            cols = (tcs[:, None] * 16 + np.arange(16)[None, :]).ravel()
+            cols = cols[cols < N]
+            rows += [cols[rng.random(len(cols)) < rng.choice([1.0, 0.5])] for _ in range(16)]
+        else:
+            c = np.sort(rng.choice(N, int(rng.integers(2, 40)), replace=False))
+            if rng.random() < 0.5:
+                c = c[::-1].copy()
+            else:
+                c[1] = c[0]
+            rows.append(c)
+    M = len(rows)
+    lens = np.array([len(r) for r in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    return M, N, K, dt, rowptr, col, val, A, B
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_similarity_mixtures(engine_factory, seed):
+    M, N, K, dt, rowptr, col, val, A, B = build_similarity_case(seed)
+    e = engine_factory()
+    if dt == "bf16":
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K)
+        e.set_dense(Ab, Bb, capi.BF16)
+    elif dt == "f16":
+        Ab, Bb = capi.to_f16(A).reshape(M, K), capi.to_f16(B).reshape(N, K)
+        A, B = capi.from_f16(Ab).reshape(M, K), capi.from_f16(Bb).reshape(N, K)
+        e.set_dense(Ab, Bb, capi.F16)
+    else:
+        e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    ref = O.sddmm_csr(rowptr, col, val, A, B)
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED, capi.FLAT):
+        e.plan(strategy)
+        e.run()
+        st = e.stats()
+        ok, worst, i = O.check_values(e.values(), ref, mag=mag)
+        assert ok, (seed, capi.STRATEGY_NAMES[strategy], dt, M, N, K, i, worst)
+        if st.strategy_used in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED):
+            assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == len(col), (seed, strategy)
+    e.close()
