@@ -968,7 +968,7 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
 struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
 
 template <int DT, int STEPS>
-__global__ __launch_bounds__(BLOCK) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+__global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const float *__restrict__ sval, float *__restrict__ P,
