@@ -281,6 +281,45 @@ def test_context_reuse_and_update_values(engine_factory):
     e.close()
 
 
+def test_distinct_contexts_on_distinct_threads(engine_factory):
+    """A context is single-threaded, but two contexts driven from two host threads at
+    once (each on its own stream) must not disturb each other: every result of every
+    round is checked, with a different matrix, width and strategy mix per thread."""
+    import threading
+
+    cases = {}
+    for t, (wl, K) in enumerate([("fem_banded", 32), ("mixed_density", 64), ("similar_rows", 32)]):
+        w = W.make(wl, "small", K=K)
+        cases[t] = (w, O.sddmm_csr(w.rowptr, w.col, w.sval, w.A, w.B, threads=0),
+                    O.sddmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)[1])
+    engines = {t: engine_factory() for t in cases}
+    errors = []
+
+    def drive(t):
+        try:
+            w, ref, mag = cases[t]
+            e = engines[t]
+            for rnd in range(6):
+                e.set_dense(w.A, w.B)
+                e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+                e.plan([capi.AUTO, capi.FLAT, capi.MFMA_TILE][(rnd + t) % 3])
+                e.run()
+                ok, worst, i = O.check_values(e.values(), ref, mag=mag, rtol=1e-5)
+                if not ok:
+                    errors.append("thread %d round %d: entry %d off by %.2f x tolerance" % (t, rnd, i, worst))
+                    return
+        except Exception as ex:                       # surfaced by the assert below
+            errors.append("thread %d: %r" % (t, ex))
+
+    threads = [threading.Thread(target=drive, args=(t,)) for t in cases]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(120)
+    assert not any(th.is_alive() for th in threads), "a thread did not finish"
+    assert not errors, errors
+
+
 def test_timing_entry_points(engine_factory):
     """Per-launch events and one event pair around a stream of launches: both leave
     the result intact, both report positive times, and a launch inside a stream is
