@@ -4,7 +4,11 @@
 // (A rows, indices, S values, FMAs, P stores) taken away.  What it reaches is the
 // ceiling of the box for that pattern at a given table size (L2-resident,
 // last-level-cache-resident, HBM).
-// usage: gather_probe [n rows] [table rows] [blocks] [sequential 0|1]
+// usage: gather_probe [n rows] [table rows] [blocks] [sequential 0|1] [index file]
+// With an index file (raw int32, e.g. the column array of a workload written by
+// `python -m dphpc_amd.workloads NAME --dump-col FILE`) the rows are gathered in
+// that order, n is the file's length, and the figure is the ceiling for that
+// very column stream, cache hits of popular columns included.
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
@@ -36,14 +40,31 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const uint4 *__restri
 }
 
 int main(int argc, char **argv) {
-    const long n = argc > 1 ? atol(argv[1]) : 2000000;
+    long n = argc > 1 ? atol(argv[1]) : 2000000;
     const long T = argc > 2 ? atol(argv[2]) : 30000;
     const int blocks = argc > 3 ? atoi(argv[3]) : 2048;
     const int seq = argc > 4 ? atoi(argv[4]) : 0;
-    if (n < 1 || T < 1 || T > 2147483647L || blocks < 1) { fprintf(stderr, "bad arguments\n"); return 2; }
-    std::vector<int> h((size_t)n);
-    std::mt19937_64 rng(1);
-    for (long i = 0; i < n; ++i) h[(size_t)i] = seq ? (int)(i % T) : (int)(rng() % (unsigned long)T);
+    const char *path = argc > 5 ? argv[5] : nullptr;
+    if ((!path && n < 1) || T < 1 || T > 2147483647L || blocks < 1) { fprintf(stderr, "bad arguments\n"); return 2; }
+    std::vector<int> h;
+    if (path) {
+        FILE *f = fopen(path, "rb");
+        if (!f) { fprintf(stderr, "cannot open %s\n", path); return 2; }
+        fseek(f, 0, SEEK_END);
+        n = ftell(f) / 4;
+        fseek(f, 0, SEEK_SET);
+        h.resize((size_t)n);
+        const size_t got = n > 0 ? fread(h.data(), 4, (size_t)n, f) : 0;
+        fclose(f);
+        if (n < 1 || got != (size_t)n) { fprintf(stderr, "cannot read %s\n", path); return 2; }
+        // every index is checked on the host: the kernel trusts them
+        for (long i = 0; i < n; ++i)
+            if (h[(size_t)i] < 0 || h[(size_t)i] >= T) { fprintf(stderr, "index %ld = %d outside the table\n", i, h[(size_t)i]); return 2; }
+    } else {
+        h.resize((size_t)n);
+        std::mt19937_64 rng(1);
+        for (long i = 0; i < n; ++i) h[(size_t)i] = seq ? (int)(i % T) : (int)(rng() % (unsigned long)T);
+    }
     uint4 *table = nullptr;
     int *idx = nullptr;
     unsigned *out = nullptr;
@@ -66,7 +87,7 @@ int main(int argc, char **argv) {
     CHECK(hipEventElapsedTime(&ms, a, b));
     const double us = ms * 1e3 / reps;
     printf("rows=%ld table=%ld rows (%.1f MB) blocks=%d %s: %.1f us per launch, %.1f G rows/s, %.2f TB/s gathered\n", n, T,
-           T * 128 / 1e6, blocks, seq ? "sequential" : "random", us, n / us / 1e3, n * 128.0 / us / 1e6);
+           T * 128 / 1e6, blocks, path ? "from file" : seq ? "sequential" : "random", us, n / us / 1e3, n * 128.0 / us / 1e6);
     CHECK(hipFree(table));
     CHECK(hipFree(idx));
     CHECK(hipFree(out));
