@@ -51,7 +51,7 @@ inline Dataset finish(const std::string &name, int M, int N, int K, std::vector<
 }
 
 // M x N with each position kept with probability `density`, values U[0,1)
-// (the shape of RandomWithDensityDataset, src/benchmark/dataset.hpp:206-230).
+// (the shape of RandomWithDensityDataset, src/benchmark/dataset.hpp:331-354).
 inline Dataset uniform_random(int M, int N, int K, double density, uint64_t seed) {
     std::mt19937_64 rng(seed);
     std::uniform_real_distribution<float> v(0.f, 1.f);
@@ -155,6 +155,35 @@ inline Dataset dense_tiles(int M, int N, int K, double tile_frac, uint64_t seed)
                     for (int c = 0; c < 16; ++c) t.push_back({ti * 16 + r, tj * 16 + c, v(rng)});
     if (t.empty()) t.push_back({0, 0, 1.f});
     return finish("dense_tiles", M, N, K, std::move(t), rng, false);
+}
+
+// One entry per row and per column at a random permutation, values U[0,1): the
+// shape of LatinHypercubeDataset (src/benchmark/dataset.hpp:358-378, sampler
+// src/utils/random_generator.hpp:82-107; the sampler there shuffles the row list
+// twice and leaves the columns in order, which is still a permutation matrix).
+inline Dataset latin_hypercube(int M, int K, uint64_t seed) {
+    std::mt19937_64 rng(seed);
+    std::uniform_real_distribution<float> v(0.f, 1.f);
+    std::vector<int> perm((size_t)M);
+    for (int i = 0; i < M; ++i) perm[(size_t)i] = i;
+    std::shuffle(perm.begin(), perm.end(), rng);
+    std::vector<Triplet<float>> t;
+    t.reserve((size_t)M);
+    for (int i = 0; i < M; ++i) t.push_back({perm[(size_t)i], i, v(rng)});
+    return finish("latin_hypercube", M, M, K, std::move(t), rng, false);
+}
+
+// The first floor(density * M) rows completely filled with ones, every other row
+// empty: the shape of UnbalancedDataset (src/benchmark/dataset.hpp:380-412).
+inline Dataset unbalanced(int M, int N, int K, double density, uint64_t seed) {
+    std::mt19937_64 rng(seed);
+    const int full_rows = (int)(std::min(1.0, std::max(density, 0.0)) * M);
+    std::vector<Triplet<float>> t;
+    t.reserve((size_t)full_rows * N);
+    for (int r = 0; r < full_rows; ++r)
+        for (int c = 0; c < N; ++c) t.push_back({r, c, 1.f});
+    if (t.empty()) t.push_back({0, 0, 1.f});
+    return finish("unbalanced", M, N, K, std::move(t), rng, false);
 }
 
 // Matrix Market coordinate reader with the reference's conventions

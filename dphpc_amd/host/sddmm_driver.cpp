@@ -3,6 +3,9 @@
 //
 //   sddmm_driver [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx|edges.txt] [--dim n] [--no_csv_header]
 //
+// Without --dataset the five benchmark shapes run; `latin_hypercube` and
+// `unbalanced` (the reference's other synthetic shapes) run when named.
+//
 // Prints one CSV line per run in the reference's 14-column schema
 // (src/main.cpp:356-358, src/benchmark/benchmark.hpp:95-98):
 //   competitor,dataset,mat_repr,M,N,K,NZ,total_ns,init_ns,comp_ns,cleanup_ns,
@@ -161,6 +164,9 @@ int main(int argc, char **argv) {
     if (want("fem_banded")) { Dataset d = sddmm_host::fem_banded(dim(36000, 8), K, dim(3000, 8), 49.4, seed + 2); bench_dataset(d, comps, num_runs); }
     if (want("power_law")) { Dataset d = sddmm_host::power_law(dim(2600000, 1), K, 13.85, 50000, seed + 3); bench_dataset(d, comps, num_runs); }
     if (want("mixed_density")) { Dataset d = sddmm_host::mixed_density(dim(30000, 1), K, 0.10, 1385, 0.40, seed + 4); bench_dataset(d, comps, num_runs); }
+    // the reference's other two synthetic shapes (src/benchmark/dataset.hpp:358-412): by name only
+    if (only == "latin_hypercube") { Dataset d = sddmm_host::latin_hypercube(dim(100000, 1), K, seed + 6); bench_dataset(d, comps, num_runs); }
+    if (only == "unbalanced") { Dataset d = sddmm_host::unbalanced(dim(20000, 16), dim(10000, 16), K, 0.05, seed + 7); bench_dataset(d, comps, num_runs); }
     if (want("dense_tiles")) { Dataset d = sddmm_host::dense_tiles(dim(4562, 16), dim(5761, 16), K, 0.094, seed + 5); bench_dataset(d, comps, num_runs); }
     return 0;
 }

@@ -206,6 +206,29 @@ static void cpu_cases() {
         for (const char *n : {"edges.txt", "bad.txt", "m.mtx", "p.mtx", "a.mtx"}) std::remove((base + "/" + n).c_str());
         rmdir(dir);
     }
+    {
+        CASE("latin_and_unbalanced_shapes");   // src/benchmark/dataset.hpp:358-412
+        const sddmm_host::Dataset l = sddmm_host::latin_hypercube(257, 8, 11);
+        CHECK(l.S_csr.getRows() == 257 && l.S_csr.getCols() == 257 && l.S_csr.getValues().size() == 257);
+        std::vector<int> per_col(257, 0);
+        bool one_per_row = true, moved = false;
+        for (int r = 0; r < 257; ++r) {
+            one_per_row = one_per_row && l.S_csr.getRowPositions()[r + 1] - l.S_csr.getRowPositions()[r] == 1;
+            const int c = l.S_csr.getColPositions()[r];
+            per_col[c] += 1;
+            moved = moved || c != r;
+        }
+        CHECK(one_per_row && moved);
+        CHECK(std::all_of(per_col.begin(), per_col.end(), [](int n) { return n == 1; }));
+        CHECK(std::all_of(l.S_csr.getValues().begin(), l.S_csr.getValues().end(), [](float v) { return v >= 0.f && v < 1.f; }));
+        const sddmm_host::Dataset u = sddmm_host::unbalanced(40, 24, 8, 0.26, 12);   // floor(0.26 * 40) = 10 full rows
+        CHECK(u.S_csr.getRows() == 40 && u.S_csr.getCols() == 24 && u.S_csr.getValues().size() == 240);
+        bool shape = true;
+        for (int r = 0; r <= 40; ++r) shape = shape && u.S_csr.getRowPositions()[r] == std::min(r, 10) * 24;
+        for (int j = 0; j < 240; ++j) shape = shape && u.S_csr.getColPositions()[j] == j % 24 && u.S_csr.getValues()[j] == 1.f;
+        CHECK(shape);
+        CHECK(u.S_coo.getRowPositions()[239] == 9 && u.A.getRows() == 40 && u.B.getRows() == 24);
+    }
 }
 
 // ---------------------------------------------------------------- GPU cases

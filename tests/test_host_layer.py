@@ -106,3 +106,14 @@ def test_driver_reads_snap_edge_list_like_the_reference(tmp_path):
                         for r in rows)
     p = _run([DRIVER, "--dataset", str(txt), "--dim", "100"], 60)
     assert p.returncode == 1 and "dimension" in p.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,nz", [("latin_hypercube", 5000), ("unbalanced", 49 * 496)])
+def test_driver_runs_the_reference_latin_and_unbalanced_shapes(name, nz):
+    # one entry per row and column; a block of completely filled leading rows
+    # (src/benchmark/dataset.hpp:358-412); scale 0.05: 5000 x 5000 and 992 x 496 with 49 full rows
+    p = _run([DRIVER, "--dataset", name, "--scale", "0.05", "--num_runs", "1", "--K", "32"], 60)
+    assert p.returncode == 0, p.stdout
+    rows = _csv_rows(p.stdout)
+    assert len(rows) == 14 and all(r["dataset"] == name and r["NZ"] == str(nz) and r["correctness"] == "1" for r in rows)
