@@ -21,7 +21,7 @@ OK, ERR_INVALID, ERR_NULL, ERR_STATE, ERR_ALLOC, ERR_HIP, ERR_UNSUPPORTED, ERR_N
 
 # every symbol include/sddmm_amd.h declares
 EXPORTS = [
-    "sddmm_create", "sddmm_destroy", "sddmm_strerror", "sddmm_last_error",
+    "sddmm_create", "sddmm_destroy", "sddmm_strerror", "sddmm_last_error", "sddmm_set_stream", "sddmm_get_stream",
     "sddmm_set_dense", "sddmm_set_dense_device", "sddmm_set_csr", "sddmm_set_coo",
     "sddmm_set_csr_device", "sddmm_update_values", "sddmm_plan", "sddmm_run",
     "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_run_fused",
@@ -76,6 +76,8 @@ def load_library():
     L.sddmm_strerror.restype = C.c_char_p
     L.sddmm_last_error.argtypes = [vp]
     L.sddmm_last_error.restype = C.c_char_p
+    L.sddmm_set_stream.argtypes = [vp, vp, i32]
+    L.sddmm_get_stream.argtypes = [vp, C.POINTER(vp)]
     L.sddmm_set_dense.argtypes = [vp, i32, i32, i32, vp, vp, i32]
     L.sddmm_set_dense_device.argtypes = [vp, i32, i32, i32, vp, vp, i32]
     L.sddmm_set_csr.argtypes = [vp, i32, i32, i64, vp, vp, vp]
@@ -198,6 +200,16 @@ class Engine:
         sval = np.ascontiguousarray(sval, np.float32)
         assert len(sval) == self.nnz
         self._chk(self.L.sddmm_update_values(self.h, _ptr(sval)))
+
+    def set_stream(self, stream, lent=True):
+        """stream: a hipStream_t as an integer (0 = the null stream); lent=False
+        returns to the context's own stream."""
+        self._chk(self.L.sddmm_set_stream(self.h, C.c_void_p(stream or None), 1 if lent else 0))
+
+    def get_stream(self):
+        p = C.c_void_p()
+        self._chk(self.L.sddmm_get_stream(self.h, C.byref(p)))
+        return p.value or 0
 
     def plan(self, strategy=AUTO):
         self._chk(self.L.sddmm_plan(self.h, strategy))

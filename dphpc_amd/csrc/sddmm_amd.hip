@@ -27,7 +27,9 @@ using namespace sddmm;
 // ---------------------------------------------------------------------------
 struct sddmm_ctx {
     int device = 0;
-    hipStream_t stream = nullptr;
+    hipStream_t stream = nullptr;      // where work is enqueued: own_stream unless the caller lent one
+    hipStream_t own_stream = nullptr;
+    bool lent_stream = false;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 
     char err[512] = {0};
@@ -979,26 +981,43 @@ int sddmm_create(sddmm_ctx **out, int device) {
     sddmm_ctx *c = new (std::nothrow) sddmm_ctx();
     if (!c) return SDDMM_ERR_ALLOC;
     c->device = device;
-    if (hipStreamCreate(&c->stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
+    if (hipStreamCreate(&c->own_stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
         hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(DevCounters)) != hipSuccess) {
         sddmm_destroy(c);
         return SDDMM_ERR_HIP;
     }
+    c->stream = c->own_stream;
     *out = c;
+    return SDDMM_OK;
+}
+
+int sddmm_set_stream(sddmm_ctx *c, void *stream, int lent) {
+    if (!c) return SDDMM_ERR_NULL;
+    HIP_TRY(c, hipSetDevice(c->device));
+    // nothing of this context may still be in flight on the stream it leaves
+    HIP_TRY(c, hipStreamSynchronize(c->stream));
+    c->lent_stream = lent != 0;
+    c->stream = c->lent_stream ? (hipStream_t)stream : c->own_stream;
+    return SDDMM_OK;
+}
+
+int sddmm_get_stream(const sddmm_ctx *c, void **stream) {
+    if (!c || !stream) return SDDMM_ERR_NULL;
+    *stream = (void *)c->stream;
     return SDDMM_OK;
 }
 
 void sddmm_destroy(sddmm_ctx *c) {
     if (!c) return;
     (void)hipSetDevice(c->device);
-    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    if (c->own_stream) (void)hipStreamSynchronize(c->stream);
     release_dense(c);
     release_sparse(c);
     dfree(c->dO);
     dfree(c->d_pc);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
-    if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
     delete c;
 }
 

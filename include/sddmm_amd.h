@@ -114,6 +114,19 @@ const char *sddmm_strerror(int code);
 /* Text of the last failure on this context ("" if none); owned by the context. */
 const char *sddmm_last_error(const sddmm_ctx *ctx);
 
+/* Every context enqueues its copies and kernels on a stream of its own (the
+ * reference's competitors launch on the null stream, e.g.
+ * src/competitors/gpu/gpu_basic.cu:83,95).
+ * lent != 0: from now on enqueue on `stream` instead, a hipStream_t of this
+ * context's device that the caller keeps alive (NULL is the device's null stream);
+ * producers of borrowed device operands and consumers of sddmm_get_values_device
+ * ordered on that stream then need no host synchronisation around sddmm_launch.
+ * lent == 0: back to the context's own stream (`stream` is ignored).  The call
+ * waits for the work of this context that is still in flight. */
+int sddmm_set_stream(sddmm_ctx *ctx, void *stream, int lent);
+/* The hipStream_t in use. */
+int sddmm_get_stream(const sddmm_ctx *ctx, void **stream);
+
 /* ---- operands (init phase) ---------------------------------------------- */
 /* A: M*K elements, B: N*K elements, row-major, leading dimension K
  * (src/matrices/Dense.hpp:43-50).  K >= 1; any K is accepted for SDDMM_F32

@@ -116,3 +116,69 @@ def test_operand_beyond_4gib_uses_64bit_offsets(engine_factory):
         ok, worst, i = O.check_values(got, ref, mag=mag)
         assert ok, (capi.STRATEGY_NAMES[strategy], i, got[i], ref[i])
     e.close()
+
+
+class _DeviceArray:
+    """A device address as something torch.as_tensor can wrap without a copy."""
+
+    def __init__(self, ptr, n, typestr="<f4"):
+        self.__cuda_array_interface__ = {"shape": (n,), "typestr": typestr, "data": (ptr, False), "version": 2}
+
+
+def test_lent_stream_orders_producers_launch_and_consumers(engine_factory):
+    """The context enqueues on a stream the caller lends (torch's here): operands
+    rewritten on that stream right before sddmm_launch, and P copied on that stream
+    right after it, need no host synchronisation in between."""
+    import torch
+
+    rng = np.random.default_rng(52)
+    M, N, K = 3000, 2500, 64
+    lens = rng.integers(0, 120, M)
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate([np.sort(rng.choice(N, size=int(l), replace=False)) for l in lens]).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    dev = torch.device("cuda:0")
+    tA, tB = torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev)
+    t_rp, t_col, t_val = torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), torch.from_numpy(val).to(dev)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream(device=dev)
+    e = engine_factory()
+    own = e.get_stream()
+    assert own != 0
+    e.set_stream(stream.cuda_stream)
+    assert e.get_stream() == stream.cuda_stream
+    L = e.L
+    e._chk(L.sddmm_set_dense_device(e.h, M, N, K, C.c_void_p(tA.data_ptr()), C.c_void_p(tB.data_ptr()), capi.F32))
+    e._chk(L.sddmm_set_csr_device(e.h, M, N, len(col), C.c_void_p(t_rp.data_ptr()), C.c_void_p(t_col.data_ptr()),
+                                  C.c_void_p(t_val.data_ptr())))
+    e.nnz = len(col)
+    e.plan(capi.AUTO)
+    dP = C.c_void_p()
+    e._chk(L.sddmm_get_values_device(e.h, C.byref(dP)))
+    tP = torch.as_tensor(_DeviceArray(dP.value, len(col)), device=dev)
+    outs = []
+    with torch.cuda.stream(stream):
+        for step in range(3):
+            # producers: a chain of updates of the borrowed operands on the lent stream
+            for _ in range(20):
+                tA.mul_(1.01)
+                tB.add_(0.001)
+            e.launch()                        # no host synchronisation on either side
+            outs.append((tA.clone(), tB.clone(), tP.clone()))
+    stream.synchronize()
+    for a, b, p in outs:
+        a, b, p = a.cpu().numpy(), b.cpu().numpy(), p.cpu().numpy()
+        ref = O.sddmm_csr(rowptr, col, val, a, b)
+        _, mag = O.sddmm_csr_f64(rowptr, col, val, a, b)
+        ok, worst, i = O.check_values(p, ref, mag=mag)
+        assert ok, (i, p[i], ref[i], worst)
+    assert not np.array_equal(outs[0][2].cpu().numpy(), outs[2][2].cpu().numpy())
+    # the null stream, then back to the context's own stream
+    for lend, handle in ((True, 0), (False, 0)):
+        e.set_stream(handle, lent=lend)
+        assert e.get_stream() == (0 if lend else own)
+        e.run()
+        np.testing.assert_array_equal(e.values(), outs[2][2].cpu().numpy())
+    e.close()
