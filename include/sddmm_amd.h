@@ -159,7 +159,9 @@ int sddmm_plan(sddmm_ctx *ctx, int strategy);
 /* Launch and wait.  P is complete on return (every reference run_csr ends in a
  * device synchronise, e.g. src/competitors/gpu/gpu_basic.hpp:72). */
 int sddmm_run(sddmm_ctx *ctx);
-/* Enqueue on the context's stream without waiting / wait for it. */
+/* Enqueue on the context's stream without waiting / wait for it.  On a planned
+ * context sddmm_launch only enqueues kernels (no allocation, copy, fill or wait), so
+ * it may be recorded into a HIP graph on a lent stream under capture. */
 int sddmm_launch(sddmm_ctx *ctx);
 int sddmm_synchronize(sddmm_ctx *ctx);
 /* warmup untimed launches, then reps launches each bracketed by HIP events on the
