@@ -85,7 +85,7 @@ struct sddmm_ctx {
     size_t sort_tmp_bytes = 0;
     int64_t cand_cap = 0, vstrips_cap = 0, n_cand = 0, n_vstrips = 0;
     unsigned int *d_vstrip_ntiles = nullptr, *d_vstrip_off = nullptr;
-    // row ownership (one byte per row: 0 row kernels, 1 dense tiles, 2 row panels, 3 gathered strips)
+    // row ownership (one byte per row: 0 row kernels, 1 dense tiles, 2 row panels, 3 gathered strips, 4 union strips)
     unsigned char *d_owner = nullptr;
     int64_t owner_cap = 0;
     bool owner_active = false;
@@ -1208,7 +1208,8 @@ int sddmm_launch(sddmm_ctx *c) {
     int rc = check_ready(c);
     if (rc) return rc;
     if (!c->planned) {
-        rc = sddmm_plan(c, SDDMM_AUTO);
+        // operands were replaced since the last plan: plan again as last asked (AUTO on a new context)
+        rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
     }
     return enqueue_run(c);
@@ -1227,7 +1228,8 @@ int sddmm_run(sddmm_ctx *c) {
     int rc = check_ready(c);
     if (rc) return rc;
     if (!c->planned) {
-        rc = sddmm_plan(c, SDDMM_AUTO);
+        // operands were replaced since the last plan: plan again as last asked (AUTO on a new context)
+        rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
     }
     HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
@@ -1362,7 +1364,8 @@ int sddmm_time_runs(sddmm_ctx *c, int warmup, int reps, int include_plan, float 
     int rc = check_ready(c);
     if (rc) return rc;
     if (!c->planned) {
-        rc = sddmm_plan(c, SDDMM_AUTO);
+        // operands were replaced since the last plan: plan again as last asked (AUTO on a new context)
+        rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
     }
     const int requested = c->requested;
@@ -1390,7 +1393,8 @@ int sddmm_time_region(sddmm_ctx *c, int reps, int include_plan, float *total_ms)
     int rc = check_ready(c);
     if (rc) return rc;
     if (!c->planned) {
-        rc = sddmm_plan(c, SDDMM_AUTO);
+        // operands were replaced since the last plan: plan again as last asked (AUTO on a new context)
+        rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
     }
     const int requested = c->requested;

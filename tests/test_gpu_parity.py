@@ -281,6 +281,28 @@ def test_context_reuse_and_update_values(engine_factory):
     e.close()
 
 
+def test_replaced_operands_are_planned_again_as_last_asked(engine_factory):
+    rng = np.random.default_rng(14)
+    e = engine_factory()
+    rowptr, col, val, A, B = _random_case(rng, 200, 150, 32, 0.3)
+    e.set_dense(A, B)
+    e.set_csr(200, 150, rowptr, col, val)
+    e.run()                                           # never planned: AUTO
+    assert e.stats().strategy_used in (capi.AUTO, capi.FLAT)
+    assert_parity(e.values(), rowptr, col, val, A, B)
+    e.plan(capi.ROW_WAVE)
+    for M, N, K in [(90, 300, 16), (400, 60, 32)]:
+        rowptr, col, val, A, B = _random_case(rng, M, N, K, 0.25)
+        e.set_dense(A, B)
+        e.set_csr(M, N, rowptr, col, val)             # drops the plan
+        e.launch()
+        e.synchronize()
+        assert_parity(e.values(), rowptr, col, val, A, B)
+        e.run()
+        assert e.stats().strategy_used == capi.ROW_WAVE
+    e.close()
+
+
 def test_distinct_contexts_on_distinct_threads(engine_factory):
     """A context is single-threaded, but two contexts driven from two host threads at
     once (each on its own stream) must not disturb each other: every result of every
