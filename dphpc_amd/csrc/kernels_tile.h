@@ -953,11 +953,14 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
 //   * B:   load lane l reads gathered row l>>2, unit 4s + (l&3): 16 segments per
 //          instruction instead of the 64 a load in operand layout would touch;
 //          operand lane (n,q) then takes its unit from load lane 4n+q;
-//   * S,P: lane l < 32 reads / writes the four consecutive entries 4(l&3).. of row
-//          l>>2 as one 16-byte access (rows start at arbitrary 4-byte offsets; global
-//          16-byte accesses need no more alignment than that): 8 rows x 64 bytes per
-//          instruction; the accumulator is moved into that layout (lane l takes from
-//          result lane 16(l&3) + (l>>2)) and multiplied by S there.
+//   * S,P: two groups of 16 columns share one access: lane l reads / writes the four
+//          consecutive entries 4(l&7).. (of the 32) of row l>>3 as one 16-byte access
+//          (rows start at arbitrary 4-byte offsets; global 16-byte accesses need no
+//          more alignment than that): 8 rows x 128 bytes per instruction.  Lanes 8..15
+//          of every 16 hold the panel's rows a second time, so the second group's
+//          results are already in place there: a select merges the two accumulators,
+//          the merged one is moved into the memory layout (lane l takes from result
+//          lane 16(l&3) + (l>>3) + 8((l>>2)&1)) and multiplied by S there.
 //
 // Pipeline: the entries are walked in chunks of 64 = 4 groups of 16 columns.  While
 // chunk c computes, the B units and S values of chunk c+1 are in flight (a group is
@@ -987,7 +990,10 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
     const int n = lane & 15, q = lane >> 4;          // operand / result layout
     const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: row, 16-byte unit inside 64 bytes
     const int to_operand_from = (4 * n + q) << 2;    // ds_bpermute address: operand lane (n,q) <- memory lane 4n+q
-    const int to_memory_from = (16 * lunit + (lrow & 7)) << 2;   // memory lane l <- result lane (row l>>2, q = l&3)
+    // S/P layout of a pair of groups: row l>>3, 16-byte unit l&7 of the 128 bytes; units 4..7 are the
+    // second group's, whose results sit in lanes 8..15 of every 16
+    const int prow = lane >> 3, punit = lane & 7;
+    const int to_memory_from = (16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
     constexpr int ROW_UNITS = STEPS * 4;
     // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
     constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
@@ -1003,8 +1009,7 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
     // the 8 rows of a panel have one length and follow each other in the CSR arrays
     const int rs0 = __builtin_amdgcn_readfirstlane(it.pad);
     const int row_len = __builtin_amdgcn_readfirstlane(rowptr[row0 + 1]) - rs0;
-    const bool mover = lane < 32;                    // lanes that read S and write P: rows 0..7
-    const int64_t out_row = (int64_t)rs0 + (int64_t)(lrow & 7) * row_len;   // this lane's S/P row starts here
+    const int64_t out_row = (int64_t)rs0 + (int64_t)prow * row_len;   // this lane's S/P row starts here
     const int last = end - 1;
     auto cols_of_chunk = [&](int base) {                        // column of entry base + lane (clamped)
         const int e = base + lane < last ? base + lane : last;
@@ -1020,12 +1025,15 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
         const uint4 *src = Bu + (int64_t)c * ROW_UNITS + lunit;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
-        // S values of entries g0+4*lunit .. +3 of this lane's row.  The window is clamped
-        // into the row (rows of a panel hold at least 4 entries); a clamped window is
-        // only ever read for the tail group, which fetches its S values again.
-        const int e = g0 + 4 * lunit < row_len - 4 ? g0 + 4 * lunit : row_len - 4;
+        // The first group of a pair also brings the S values of entries g0+4*punit .. +3 of
+        // this lane's row, for both groups.  The window is clamped into the row (rows of a
+        // panel hold at least 4 entries); a clamped window is never used: lanes whose four
+        // entries are not all inside the item fetch their S values again.
         o.s = F4u{0.f, 0.f, 0.f, 0.f};
-        if (mover) o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
+        if ((u & 1) == 0) {
+            const int e = g0 + 4 * punit < row_len - 4 ? g0 + 4 * punit : row_len - 4;
+            o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
+        }
         return o;
     };
     auto permute4 = [&](int from, uint32_t x, uint32_t y, uint32_t z, uint32_t w_) {
@@ -1036,8 +1044,7 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
         r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)w_);
         return r;
     };
-    auto compute_store = [&](const Oper &o, int g0) {
-        if (g0 >= end) return;                                   // wave-uniform
+    auto compute = [&](const Oper &o) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
@@ -1059,27 +1066,35 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
                                                            __builtin_bit_cast(float, a[s].w), acc, 0, 0, 0);
             }
         }
-        // result lane (n,q) holds entries g0+4q.. of row n; memory lane l wants row l>>2,
-        // entries g0+4(l&3)..
+        return acc;
+    };
+    // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
+    auto compute_store_pair = [&](const Oper &o0, const Oper &o1, int g0) {
+        if (g0 >= end) return;                                   // wave-uniform
+        const f32x4_t acc0 = compute(o0);
+        const f32x4_t acc1 = compute(o1);                        // columns clamped past the end: computed, not stored
+        // result lane (n,q) holds entries 4q.. of its group for row n&7: lanes with n < 8 keep
+        // the first group's, lanes with n >= 8 the second group's; memory lane l wants row l>>3,
+        // entries g0+4(l&7)..
         // (element values first: a bit cast applied to a vector element expression reads element 0)
-        const float r0 = acc[0], r1 = acc[1], r2 = acc[2], r3 = acc[3];
+        const bool second = (n & 8) != 0;
+        const float r0 = second ? acc1[0] : acc0[0], r1 = second ? acc1[1] : acc0[1];
+        const float r2 = second ? acc1[2] : acc0[2], r3 = second ? acc1[3] : acc0[3];
         const uint4 m = permute4(to_memory_from, __builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1),
                                  __builtin_bit_cast(uint32_t, r2), __builtin_bit_cast(uint32_t, r3));
         const float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
         const float d2 = __builtin_bit_cast(float, m.z), d3 = __builtin_bit_cast(float, m.w);
-        if (mover) {
-            const int e = g0 + 4 * lunit;
-            if (g0 + 16 <= end) {
-                // full group: four consecutive entries per lane
-                F4u out{d0 * o.s.x, d1 * o.s.y, d2 * o.s.z, d3 * o.s.w};
-                *reinterpret_cast<F4u *>(P + out_row + e) = out;
-            } else {
-                // tail group: the S values were read from a clamped window, fetch them again
-                const float d[4] = {d0, d1, d2, d3};
+        const int e = g0 + 4 * punit;
+        if (e + 4 <= end) {
+            // four consecutive entries inside the item (so the S window was not clamped)
+            F4u out{d0 * o0.s.x, d1 * o0.s.y, d2 * o0.s.z, d3 * o0.s.w};
+            *reinterpret_cast<F4u *>(P + out_row + e) = out;
+        } else {
+            // the item ends inside these four: entry by entry, S values fetched again
+            const float d[4] = {d0, d1, d2, d3};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (e + i < end) P[out_row + e + i] = d[i] * sval[out_row + e + i];
-            }
+            for (int i = 0; i < 4; ++i)
+                if (e + i < end) P[out_row + e + i] = d[i] * sval[out_row + e + i];
         }
     };
 
@@ -1101,9 +1116,10 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
     for (int base = start; base < end; base += CHUNK) {
         const int cc_nn = cols_of_chunk(base + 2 * CHUNK);
 #pragma unroll
-        for (int u = 0; u < GROUPS; ++u) {
-            compute_store(o[u], base + 16 * u);
+        for (int u = 0; u < GROUPS; u += 2) {
+            compute_store_pair(o[u], o[u + 1], base + 16 * u);
             o[u] = load_oper(cc_nxt, u, base + CHUNK + 16 * u);
+            o[u + 1] = load_oper(cc_nxt, u + 1, base + CHUNK + 16 * u + 16);
         }
         cc_nxt = cc_nn;
     }
