@@ -606,7 +606,7 @@ def test_row_panels(engine_factory, monkeypatch, K, dtype):
         for _ in range(n_rows):
             rows_cols.append(cols.copy())
 
-    add_group(8, 300)          # rows 0-7    panel, several segments
+    add_group(8, 300)          # rows 0-7    panel (several work items when SDDMM_PANEL_SEG is small)
     add_group(8, 70)           # rows 8-15   panel
     add_group(3, 40)           # rows 16-18  too few rows ...
     add_group(8, 40)           # rows 19-26  ... and this group is not 8-aligned
@@ -648,6 +648,14 @@ def test_row_panels(engine_factory, monkeypatch, K, dtype):
             exp = [(0, 300), (8, 70), (32, 33), (40, 33), (56, 9)] if applicable else []
             assert st.panels == len(exp) and st.nnz_panel == sum(8 * l for _, l in exp)
             assert st.mfma_tiles == 0
+            st_lds = st
+    # column lists cut into several work items, at boundaries that are and are not multiples of 4
+    for seg in ("96", "100", "67"):
+        monkeypatch.setenv("SDDMM_PANEL_SEG", seg)
+        got, st2 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.LDS_TILED, dt)
+        assert_parity(got, rowptr, col, val, A, B, what="panels K=%d in segments of %s" % (K, seg))
+        assert st2.panels == st_lds.panels and st2.nnz_panel == st_lds.nnz_panel
+    monkeypatch.delenv("SDDMM_PANEL_SEG")
     monkeypatch.setenv("SDDMM_PANEL_MFMA", "0")
     lds, st = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.LDS_TILED, dt)
     assert_parity(lds, rowptr, col, val, A, B, what="VALU panels K=%d" % K)
