@@ -1064,6 +1064,12 @@ __global__ __launch_bounds__(BLOCK, STEPS == 8 ? 4 : 1) void k_panel_mfma(const 
                                                            __builtin_bit_cast(float, a[s].z), acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, b.w),
                                                            __builtin_bit_cast(float, a[s].w), acc, 0, 0, 0);
+                // Order of issue: the four permutes of a step, then its four MFMAs.  Left alone the
+                // compiler pairs every MFMA with one permute and a wait for it (16 LDS round trips
+                // per 16 columns in the wave's dependency chain instead of 4); whole groups of 8 or
+                // 16 permutes ahead of their MFMAs were measured slower than either.
+                __builtin_amdgcn_sched_group_barrier(0x080, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
             }
         }
         return acc;
