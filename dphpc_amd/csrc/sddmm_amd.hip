@@ -693,8 +693,9 @@ void launch_panel_u(sddmm_ctx *c, const Shape &s) {
 }
 template <int DT, int STEPS>
 void launch_panel_mfma_t(sddmm_ctx *c) {
-    const int64_t nblocks = (c->n_panel_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_panel_mfma<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+    constexpr int PW = panel_mfma_waves(STEPS);
+    const int64_t nblocks = (c->n_panel_items + PW - 1) / PW;
+    hipLaunchKernelGGL((k_panel_mfma<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(PW * WAVE), 0, c->stream,
                        (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
                        c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
 }
