@@ -23,7 +23,7 @@ OK, ERR_INVALID, ERR_NULL, ERR_STATE, ERR_ALLOC, ERR_HIP, ERR_UNSUPPORTED, ERR_N
 EXPORTS = [
     "sddmm_create", "sddmm_destroy", "sddmm_strerror", "sddmm_last_error", "sddmm_set_stream", "sddmm_get_stream",
     "sddmm_set_dense", "sddmm_set_dense_device", "sddmm_set_csr", "sddmm_set_coo",
-    "sddmm_set_csr_device", "sddmm_update_values", "sddmm_plan", "sddmm_run",
+    "sddmm_set_csr_device", "sddmm_set_coo_device", "sddmm_update_values", "sddmm_plan", "sddmm_run",
     "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_run_fused",
     "sddmm_get_fused", "sddmm_get_fused_device", "sddmm_get_values",
     "sddmm_get_values_device", "sddmm_last_stats", "sddmm_partition_rows", "sddmm_version",
@@ -83,6 +83,7 @@ def load_library():
     L.sddmm_set_csr.argtypes = [vp, i32, i32, i64, vp, vp, vp]
     L.sddmm_set_coo.argtypes = [vp, i32, i32, i64, vp, vp, vp]
     L.sddmm_set_csr_device.argtypes = [vp, i32, i32, i64, vp, vp, vp]
+    L.sddmm_set_coo_device.argtypes = [vp, i32, i32, i64, vp, vp, vp]
     L.sddmm_update_values.argtypes = [vp, vp]
     L.sddmm_plan.argtypes = [vp, i32]
     L.sddmm_run.argtypes = [vp]

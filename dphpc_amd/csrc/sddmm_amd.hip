@@ -1107,27 +1107,36 @@ int sddmm_set_csr_device(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t 
     return SDDMM_OK;
 }
 
-int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, const int32_t *col,
-                  const float *sval) {
+static int set_coo_common(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, const int32_t *col,
+                          const float *sval, bool on_device) {
     if (!c) return SDDMM_ERR_NULL;
     HIP_TRY(c, hipSetDevice(c->device));
     int rc = check_dims(c, M, N, nnz);
     if (rc) return rc;
     if (nnz > 0 && (!row || !col || !sval)) return fail(c, SDDMM_ERR_NULL, "row, col or values is NULL");
     release_sparse(c);
-    c->own_sparse = c->own_rowptr = c->own_rowidx = true;
+    c->own_sparse = c->own_rowidx = !on_device;
+    c->own_rowptr = true;                 // the row pointer is always built here
     c->from_coo = true;
-    ALLOC_TRY(c, c->d_rowidx, (size_t)nnz * sizeof(int32_t));
-    ALLOC_TRY(c, c->d_col, (size_t)nnz * sizeof(int32_t));
-    ALLOC_TRY(c, c->d_sval, (size_t)nnz * sizeof(float));
+    if (on_device) {
+        c->d_rowidx = const_cast<int32_t *>(row);
+        c->d_col = const_cast<int32_t *>(col);
+        c->d_sval = const_cast<float *>(sval);
+    } else {
+        ALLOC_TRY(c, c->d_rowidx, (size_t)nnz * sizeof(int32_t));
+        ALLOC_TRY(c, c->d_col, (size_t)nnz * sizeof(int32_t));
+        ALLOC_TRY(c, c->d_sval, (size_t)nnz * sizeof(float));
+    }
     ALLOC_TRY(c, c->dP, (size_t)nnz * sizeof(float));
     ALLOC_TRY(c, c->d_rowptr, (size_t)(M + 1) * sizeof(int32_t));
     c->sM = M; c->sN = N; c->nnz = nnz;
     HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
     if (nnz) {
-        HIP_TRY(c, hipMemcpyAsync(c->d_rowidx, row, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
-        HIP_TRY(c, hipMemcpyAsync(c->d_col, col, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
-        HIP_TRY(c, hipMemcpyAsync(c->d_sval, sval, (size_t)nnz * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        if (!on_device) {
+            HIP_TRY(c, hipMemcpyAsync(c->d_rowidx, row, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+            HIP_TRY(c, hipMemcpyAsync(c->d_col, col, (size_t)nnz * sizeof(int32_t), hipMemcpyHostToDevice, c->stream));
+            HIP_TRY(c, hipMemcpyAsync(c->d_sval, sval, (size_t)nnz * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        }
         HIP_TRY(c, hipMemsetAsync(c->dP, 0, (size_t)nnz * sizeof(float), c->stream));
         const int g = grid_capped(nnz, 256);
         hipLaunchKernelGGL(k_check_index, dim3(g), dim3(256), 0, c->stream, c->d_rowidx, nnz, M, c->d_pc);
@@ -1165,6 +1174,15 @@ int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, c
     }
     c->have_sparse = true;
     return SDDMM_OK;
+}
+
+int sddmm_set_coo(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *row, const int32_t *col,
+                  const float *sval) {
+    return set_coo_common(c, M, N, nnz, row, col, sval, false);
+}
+int sddmm_set_coo_device(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t *d_row, const int32_t *d_col,
+                         const float *d_sval) {
+    return set_coo_common(c, M, N, nnz, d_row, d_col, d_sval, true);
 }
 
 int sddmm_update_values(sddmm_ctx *c, const float *sval) {

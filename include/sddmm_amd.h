@@ -149,6 +149,10 @@ int sddmm_set_coo(sddmm_ctx *ctx, int M, int N, int64_t nnz,
 /* Device-resident CSR (borrowed).  The structure is validated on the device. */
 int sddmm_set_csr_device(sddmm_ctx *ctx, int M, int N, int64_t nnz,
                          const int32_t *d_rowptr, const int32_t *d_col, const float *d_sval);
+/* Device-resident COO (borrowed), same rules as sddmm_set_coo; the row pointer of
+ * row-sorted input is built by the context. */
+int sddmm_set_coo_device(sddmm_ctx *ctx, int M, int N, int64_t nnz,
+                         const int32_t *d_row, const int32_t *d_col, const float *d_sval);
 /* Replace the S values only (same pattern), e.g. between iterations of a solver. */
 int sddmm_update_values(sddmm_ctx *ctx, const float *sval);
 

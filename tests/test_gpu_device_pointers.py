@@ -85,6 +85,56 @@ def test_device_resident_operands(engine_factory):
         hip.free_all()
 
 
+def test_device_resident_coo(engine_factory):
+    """Borrowed COO arrays: row-sorted input gets a row pointer (every strategy), shuffled
+    input keeps its entry order on FLAT / EXACT; bad indices are found on the device."""
+    rng = np.random.default_rng(54)
+    M, N, K = 400, 350, 32
+    mask = rng.random((M, N)) < 0.08
+    r, c = np.nonzero(mask)
+    r, c = r.astype(np.int32), c.astype(np.int32)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r, c, v)
+    ref = O.sddmm_csr(rowptr, col, val, A, B)
+    _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
+    hip = Hip()
+    e = engine_factory()
+    try:
+        L = e.L
+        e.set_dense(A, B)
+        d_r, d_c, d_v = hip.upload(r), hip.upload(c), hip.upload(v)
+        e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r, d_c, d_v))
+        e.nnz = len(r)
+        for strategy in (capi.AUTO, capi.ROW_WAVE, capi.FLAT, capi.MFMA_TILE, capi.EXACT):
+            e.plan(strategy)
+            e.run()
+            assert O.check_values(e.values(), ref, mag=mag)[0], capi.STRATEGY_NAMES[strategy]
+        with pytest.raises(capi.SddmmError):
+            e.update_values(v)                       # borrowed values
+        perm = rng.permutation(len(r))
+        d_r2, d_c2, d_v2 = hip.upload(r[perm]), hip.upload(c[perm]), hip.upload(v[perm])
+        e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r2, d_c2, d_v2))
+        for strategy in (capi.AUTO, capi.FLAT, capi.EXACT):
+            e.plan(strategy)
+            e.run()
+            got = e.values()
+            assert e.stats().strategy_used in (capi.FLAT, capi.EXACT)
+            assert O.check_values(got, ref[perm], mag=mag[perm])[0]
+        with pytest.raises(capi.SddmmError) as ei:
+            e.plan(capi.ROW_WAVE)                    # needs row-sorted entries
+        assert ei.value.code == capi.ERR_UNSUPPORTED
+        bad = r.copy()
+        bad[3] = M
+        d_bad = hip.upload(bad)
+        assert L.sddmm_set_coo_device(e.h, M, N, len(r), d_bad, d_c, d_v) == capi.ERR_PATTERN
+        assert L.sddmm_set_coo_device(e.h, M, N, len(r), None, d_c, d_v) == capi.ERR_NULL
+    finally:
+        e.close()
+        hip.free_all()
+
+
 def test_operand_beyond_4gib_uses_64bit_offsets(engine_factory):
     """B of 4 GiB + a little: rows near the end sit beyond a 32-bit byte offset."""
     K = 32
