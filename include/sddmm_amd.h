@@ -137,7 +137,8 @@ int sddmm_set_dense(sddmm_ctx *ctx, int M, int N, int K, const void *A, const vo
 int sddmm_set_dense_device(sddmm_ctx *ctx, int M, int N, int K, const void *dA, const void *dB, int dtype);
 
 /* CSR as in src/matrices/CSR.hpp:162-167: rowptr[M+1] non-decreasing with rowptr[0]==0
- * and rowptr[M]==nnz, col[nnz] in [0,N).  Columns need not be sorted; duplicates are
+ * and rowptr[M]==nnz, col[nnz] in [0,N); nnz <= 2^31 - 2^16 (32-bit positions like the
+ * reference's, with room for the kernels' look-ahead).  Columns need not be sorted; duplicates are
  * computed independently.  Violations return SDDMM_ERR_PATTERN. */
 int sddmm_set_csr(sddmm_ctx *ctx, int M, int N, int64_t nnz,
                   const int32_t *rowptr, const int32_t *col, const float *sval);

@@ -244,6 +244,10 @@ def test_error_paths_on_device(engine_factory):
     with pytest.raises(capi.SddmmError) as ei:
         e.set_coo(4, 5, np.array([0, 4], np.int32), np.array([0, 0], np.int32), np.ones(2, f32))
     assert ei.value.code == capi.ERR_PATTERN
+    # more entries than 32-bit positions (with look-ahead room) hold: refused before any array is read
+    tiny = np.zeros(8, np.int32)
+    assert e.L.sddmm_set_csr(e.h, 4, 5, 2 ** 31 - 1000, capi._ptr(tiny), capi._ptr(tiny),
+                             capi._ptr(tiny.view(f32))) == capi.ERR_INVALID
     # S larger than the dense operands
     e.set_csr(6, 5, np.zeros(7, np.int32), np.zeros(0, np.int32), np.zeros(0, f32))
     with pytest.raises(capi.SddmmError) as ei:
