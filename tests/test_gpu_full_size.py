@@ -58,3 +58,44 @@ def test_full_size(engine_factory, name, K, other):
     e.run()
     np.testing.assert_array_equal(e.values().view(np.uint32), ref.view(np.uint32))
     e.close()
+
+
+def test_positions_beyond_2_to_the_30(engine_factory):
+    """1.2e9 stored entries: positions above 2^30, byte offsets above 4 GiB in the entry
+    arrays.  Groups of 8 identical rows, so AUTO takes the panel kernel; the exact kernel
+    must match the oracle bit for bit, the others to the usual tolerance (all values are
+    of order one here, checked in slices to keep host memory flat)."""
+    M, L, N, K = 300000, 4000, 50000, 32
+    rng = np.random.default_rng(7)
+    starts = np.repeat(rng.integers(0, 2000, M // 8), 8).astype(np.int32)
+    col = (starts[:, None] + (12 * np.arange(L, dtype=np.int32))[None, :]).reshape(-1)
+    rowptr = (np.arange(M + 1, dtype=np.int64) * L).astype(np.int32)
+    nnz = len(col)
+    assert nnz > 2 ** 30
+    val = rng.random(nnz, dtype=f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    print("entries", nnz, flush=True)
+    ref = O.sddmm_csr(rowptr, col, val, A, B, threads=0)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    step = 1 << 26
+    for strategy in (capi.EXACT, capi.AUTO, capi.FLAT):
+        print("strategy", capi.STRATEGY_NAMES[strategy], flush=True)
+        e.plan(strategy)
+        e.run()
+        got = e.values()
+        st = e.stats()
+        if strategy == capi.AUTO:
+            assert st.panels == M // 8 and st.nnz_panel == nnz
+        for i in range(0, nnz, step):
+            g, r = got[i:i + step], ref[i:i + step]
+            if strategy == capi.EXACT:
+                assert np.array_equal(g.view(np.uint32), r.view(np.uint32)), i
+            else:
+                # S in [0,1), |a b| < 1: the cancellation-free magnitude |S| sum |a b| averages 4 and the
+                # parity bar is 1e-5 * max(|ref|, magnitude / 4); 1.5e-5 absolute is at least as strict
+                assert float(np.abs(g - r).max()) <= 1.5e-5, (capi.STRATEGY_NAMES[strategy], i)
+        del got
+    e.close()
