@@ -30,6 +30,7 @@ struct sddmm_ctx {
     hipStream_t stream = nullptr;      // where work is enqueued: own_stream unless the caller lent one
     hipStream_t own_stream = nullptr;
     bool lent_stream = false;
+    bool oversize = false;             // a launch was skipped because its grid does not fit one dispatch
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 
     char err[512] = {0};
@@ -133,6 +134,33 @@ int fail(sddmm_ctx *c, int code, const char *fmt, ...) {
             return fail((c), SDDMM_ERR_ALLOC, "hipMalloc(%zu bytes) failed: %s", (size_t)(bytes), \
                         hipGetErrorString(e_));                                                  \
         }                                                                                        \
+    } while (0)
+
+// A dispatch packet counts the work-items of a grid dimension in 32 bits: a launch of 2^32
+// threads or more would run only part of its grid, without any error.  Such a launch is not
+// made; launch_status() turns the skipped launch into an error of the entry point.
+#define SDDMM_LAUNCH(c, kernel, grid, block, ...)                                                        \
+    do {                                                                                                 \
+        const int64_t g_ = (int64_t)(grid);                                                              \
+        const int b_ = (int)(block);                                                                     \
+        if (g_ * b_ >= ((int64_t)1 << 32)) (c)->oversize = true;                                         \
+        else hipLaunchKernelGGL(kernel, dim3((unsigned)g_), dim3((unsigned)b_), 0, (c)->stream, __VA_ARGS__); \
+    } while (0)
+
+int launch_status(sddmm_ctx *c) {
+    if (!c->oversize) return SDDMM_OK;
+    c->oversize = false;
+    return fail(c, SDDMM_ERR_UNSUPPORTED,
+                "a kernel of this strategy needs 2^32 threads or more in one launch for this matrix "
+                "(one wavefront per row or per work item): use SDDMM_AUTO or SDDMM_FLAT");
+}
+
+// after a group of launches: a failed launch, or one that was not made
+#define LAUNCH_CHECK(c)                                \
+    do {                                               \
+        HIP_TRY(c, hipGetLastError());                 \
+        const int ls_ = launch_status(c);              \
+        if (ls_) return ls_;                           \
     } while (0)
 
 template <class T>
@@ -287,7 +315,7 @@ void launch_flat(sddmm_ctx *c) {
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
-        hipLaunchKernelGGL((k_flat<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+        SDDMM_LAUNCH(c, (k_flat<LT>), xcd_grid(nblocks), BLOCK,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowidx, c->d_col, c->d_sval, c->dP,
                            c->nnz, cpw, nblocks);
     });
@@ -298,7 +326,7 @@ void launch_row_wave(sddmm_ctx *c, const RowItem *items, int64_t n_items) {
     const int64_t nblocks = (n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
-        hipLaunchKernelGGL((k_row_wave<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+        SDDMM_LAUNCH(c, (k_row_wave<LT>), xcd_grid(nblocks), BLOCK,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
                            items, n_items, nblocks);
     });
@@ -318,7 +346,7 @@ void launch_short_rows(sddmm_ctx *c, int ts, int rpw) {
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
-        hipLaunchKernelGGL((k_short_rows<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+        SDDMM_LAUNCH(c, (k_short_rows<LT>), xcd_grid(nblocks), BLOCK,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
                            c->sM, ts, rpw, nblocks);
     });
@@ -348,7 +376,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
         using LT = decltype(L);
         constexpr int KU_ = LT::LPN * LT::UPL;
         if constexpr (!LT::LONG && LT::FULLK && !LT::WIDE && LT::U::ELEMS > 1 && (KU_ == 4 || KU_ == 8 || KU_ == 16 || KU_ == 32 || KU_ == 64)) {
-            hipLaunchKernelGGL((k_auto_tiles<LT, KU_ / 4>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+            SDDMM_LAUNCH(c, (k_auto_tiles<LT, KU_ / 4>), xcd_grid(nblocks), BLOCK,
                                (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
                                (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
                                c->dP, c->sM, c->N, c->ts, c->rpw, short_blocks, c->d_items, c->n_items,
@@ -368,7 +396,7 @@ void launch_auto(sddmm_ctx *c) {
     const int64_t nblocks = short_blocks + item_blocks;
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
-        hipLaunchKernelGGL((k_auto<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+        SDDMM_LAUNCH(c, (k_auto<LT>), xcd_grid(nblocks), BLOCK,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
                            c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
@@ -389,11 +417,11 @@ int classify_rows(sddmm_ctx *c) {
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     if (nb > 0) {
         const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
-        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr, owner,
+        SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr, owner,
                            c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc);
-        hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
+        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
     int rc = fetch_counters(c);
     if (rc) return rc;
@@ -407,10 +435,10 @@ int classify_rows(sddmm_ctx *c) {
         c->items_cap = c->n_items;
     }
     if (c->n_items > 0) {
-        hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+        SDDMM_LAUNCH(c, k_classify_write, nb, SCAN_BLOCK, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts, c->seg,
                            c->d_block_sums, c->d_items);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
     return SDDMM_OK;
 }
@@ -423,11 +451,11 @@ int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t
         ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
         c->block_sums_cap = nb;
     }
-    hipLaunchKernelGGL(k_scan_sums, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, in, n, c->d_block_sums);
-    hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb, d_total);
-    hipLaunchKernelGGL(k_scan_apply, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, in, n,
+    SDDMM_LAUNCH(c, k_scan_sums, nb, SCAN_BLOCK, in, n, c->d_block_sums);
+    SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb, d_total);
+    SDDMM_LAUNCH(c, k_scan_apply, nb, SCAN_BLOCK, in, n,
                        (const unsigned int *)c->d_block_sums, out);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     return SDDMM_OK;
 }
 
@@ -479,9 +507,9 @@ int plan_tiles_count(sddmm_ctx *c, int min_fill) {
         c->strips_cap = n_strips;
     }
     const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-    hipLaunchKernelGGL(k_strip_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+    SDDMM_LAUNCH(c, k_strip_count, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                        c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner, c->d_pc);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     return device_scan(c, c->d_strip_ntiles, c->d_strip_off, n_strips, &c->d_pc->tiles_scanned);
 }
 
@@ -513,9 +541,9 @@ int plan_union_count(sddmm_ctx *c, int min_fill) {
         c->ustrips_cap = n_strips;
     }
     const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-    hipLaunchKernelGGL(k_union_count, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+    SDDMM_LAUNCH(c, k_union_count, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                        c->d_col, c->sM, n_strips, min_fill, c->d_owner, c->d_ustrip_ntiles, c->d_pc);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     c->union_counted = true;
     return device_scan(c, c->d_ustrip_ntiles, c->d_ustrip_off, n_strips, &c->d_pc->utiles_scanned);
 }
@@ -531,10 +559,10 @@ int plan_gathered_candidates(sddmm_ctx *c, int min_len) {
         ALLOC_TRY(c, c->d_sorted_keys, (size_t)M * sizeof(unsigned long long));
         c->cand_cap = M;
     }
-    hipLaunchKernelGGL(k_gather_candidates, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, c->stream, c->d_rowptr,
+    SDDMM_LAUNCH(c, k_gather_candidates, ((M + 255) / 256), 256, c->d_rowptr,
                        c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys,
                        &c->d_pc->n_candidates);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     return SDDMM_OK;
 }
 
@@ -563,10 +591,10 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
         ALLOC_TRY(c, c->d_vrows, (size_t)c->n_vstrips * 16 * sizeof(int32_t));
         c->vstrips_cap = c->n_vstrips;
     }
-    hipLaunchKernelGGL(k_gathered_count, dim3((unsigned)c->n_vstrips), dim3(GATHERED_BLOCK), 0, c->stream, c->d_rowptr, c->d_col,
+    SDDMM_LAUNCH(c, k_gathered_count, c->n_vstrips, GATHERED_BLOCK, c->d_rowptr, c->d_col,
                        (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
                        c->d_vrows, c->d_owner, c->d_pc);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     rc = device_scan(c, c->d_vstrip_ntiles, c->d_vstrip_off, c->n_vstrips, &c->d_pc->tiles_scanned);
     if (rc) return rc;
     rc = fetch_counters(c);
@@ -591,29 +619,29 @@ int plan_tiles_fill(sddmm_ctx *c) {
     if (c->n_tiles_natural > 0) {
         const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
         const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-        hipLaunchKernelGGL(k_strip_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+        SDDMM_LAUNCH(c, k_strip_tiles, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                            c->d_col, c->sM, n_strips, c->d_strip_ntiles, c->d_strip_off, c->d_tiles, c->d_tile_cols);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
     if (c->n_tiles_union > 0) {
         const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
         const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
-        hipLaunchKernelGGL(k_union_tiles, dim3(strip_grid), dim3(WAVE * STRIPS_PER_BLOCK), 0, c->stream, c->d_rowptr,
+        SDDMM_LAUNCH(c, k_union_tiles, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                            c->d_col, c->sM, n_strips, c->d_ustrip_ntiles, c->d_ustrip_off,
                            c->d_tiles + c->n_tiles_natural, c->d_tile_cols + c->n_tiles_natural * 16);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
     if (c->n_tiles > c->n_tiles_natural + c->n_tiles_union) {
-        hipLaunchKernelGGL(k_gathered_tiles, dim3((unsigned)c->n_vstrips), dim3(GATHERED_BLOCK), 0, c->stream, c->d_rowptr,
+        SDDMM_LAUNCH(c, k_gathered_tiles, c->n_vstrips, GATHERED_BLOCK, c->d_rowptr,
                            c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
                            c->d_vstrip_off, c->d_tiles + c->n_tiles_natural + c->n_tiles_union,
                            c->d_tile_cols + (c->n_tiles_natural + c->n_tiles_union) * 16);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
-    hipLaunchKernelGGL(k_tile_rows, dim3((unsigned)((c->n_tiles * 16 + 255) / 256)), dim3(256), 0, c->stream,
+    SDDMM_LAUNCH(c, k_tile_rows, ((c->n_tiles * 16 + 255) / 256), 256,
                        c->d_rowptr, c->d_col, c->sM, (const int32_t *)c->d_vrows, (const int32_t *)c->d_tile_cols,
                        c->d_tiles, c->n_tiles);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     c->tiles_active = true;
     c->tiles_per_wave = std::max(1, env_int("SDDMM_TPW", 4));
     return SDDMM_OK;
@@ -652,9 +680,9 @@ int plan_panels_flags(sddmm_ctx *c, int min_len, int pseg) {
         ALLOC_TRY(c, c->d_panel_off, (size_t)n_panels * sizeof(unsigned int));
         c->panels_cap = n_panels;
     }
-    hipLaunchKernelGGL(k_panel_flags, dim3((unsigned)((n_panels * WAVE + 255) / 256)), dim3(256), 0, c->stream,
+    SDDMM_LAUNCH(c, k_panel_flags, ((n_panels * WAVE + 255) / 256), 256,
                        c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner, c->d_panel_counts, c->d_pc);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     c->panels_flagged = true;
     return device_scan(c, c->d_panel_counts, c->d_panel_off, n_panels, &c->d_pc->panel_items);
 }
@@ -671,10 +699,10 @@ int plan_panels_items(sddmm_ctx *c, int pseg) {
         ALLOC_TRY(c, c->d_panel_items, (size_t)c->n_panel_items * sizeof(RowItem));
         c->panel_items_cap = c->n_panel_items;
     }
-    hipLaunchKernelGGL(k_panel_items, dim3((unsigned)((n_panels + 255) / 256)), dim3(256), 0, c->stream, c->d_rowptr,
+    SDDMM_LAUNCH(c, k_panel_items, ((n_panels + 255) / 256), 256, c->d_rowptr,
                        n_panels, pseg, (const unsigned int *)c->d_panel_counts, (const unsigned int *)c->d_panel_off,
                        c->d_panel_items);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     return SDDMM_OK;
 }
 
@@ -682,7 +710,7 @@ template <class U, int UPL>
 void launch_panel_t(sddmm_ctx *c, int KU) {
     using LT = Layout<U, 8, UPL, true, false>;
     const int64_t nblocks = (c->n_panel_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_panel<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+    SDDMM_LAUNCH(c, (k_panel<LT>), xcd_grid(nblocks), BLOCK,
                        (const void *)c->dA, (const void *)c->dB, KU, c->d_rowptr, c->d_col, c->d_sval, c->dP,
                        (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
 }
@@ -695,7 +723,7 @@ template <int DT, int STEPS>
 void launch_panel_mfma_t(sddmm_ctx *c) {
     constexpr int PW = panel_mfma_waves(STEPS);
     const int64_t nblocks = (c->n_panel_items + PW - 1) / PW;
-    hipLaunchKernelGGL((k_panel_mfma<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(PW * WAVE), 0, c->stream,
+    SDDMM_LAUNCH(c, (k_panel_mfma<DT, STEPS>), xcd_grid(nblocks), PW * WAVE,
                        (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
                        c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
 }
@@ -727,7 +755,7 @@ template <int DT, int STEPS>
 void launch_tile_t(sddmm_ctx *c) {
     const int64_t waves = (c->n_tiles + c->tiles_per_wave - 1) / c->tiles_per_wave;
     const int64_t nblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    hipLaunchKernelGGL((k_tile<DT, STEPS>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+    SDDMM_LAUNCH(c, (k_tile<DT, STEPS>), xcd_grid(nblocks), BLOCK,
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
                        (const int32_t *)c->d_tile_cols, (const TileDesc *)c->d_tiles, c->n_tiles,
                        c->tiles_per_wave, (const float *)c->d_sval, c->dP, nblocks);
@@ -753,9 +781,9 @@ int ensure_rowidx(sddmm_ctx *c) {
     ALLOC_TRY(c, c->d_rowidx, (size_t)c->nnz * sizeof(int32_t));
     c->own_rowidx = true;
     if (c->sM > 0 && c->nnz > 0)
-        hipLaunchKernelGGL(k_expand_rows, dim3(grid_for(c->sM, 256)), dim3(256), 0, c->stream, c->d_rowptr, c->sM,
+        SDDMM_LAUNCH(c, k_expand_rows, grid_for(c->sM, 256), 256, c->d_rowptr, c->sM,
                            c->d_rowidx);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     return SDDMM_OK;
 }
 
@@ -763,17 +791,17 @@ int ensure_rowidx(sddmm_ctx *c) {
 int validate_csr(sddmm_ctx *c) {
     HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
     if (c->sM > 0)
-        hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(c->sM, 256)), dim3(256), 0, c->stream, c->d_rowptr, c->sM,
+        SDDMM_LAUNCH(c, k_check_rowptr, grid_for(c->sM, 256), 256, c->d_rowptr, c->sM,
                            c->nnz, c->d_pc);
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     int rc = fetch_counters(c);
     if (rc) return rc;
     if (c->pc.bad_pattern) return fail(c, SDDMM_ERR_PATTERN, "rowptr is not a valid CSR row pointer array");
     // only now is it safe to walk col[0..nnz)
     if (c->nnz > 0) {
-        hipLaunchKernelGGL(k_check_index, dim3(grid_capped(c->nnz, 256)), dim3(256), 0, c->stream, c->d_col, c->nnz,
+        SDDMM_LAUNCH(c, k_check_index, grid_capped(c->nnz, 256), 256, c->d_col, c->nnz,
                            c->sN, c->d_pc);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
         rc = fetch_counters(c);
         if (rc) return rc;
         if (c->pc.bad_pattern) return fail(c, SDDMM_ERR_PATTERN, "column index outside [0,N)");
@@ -818,18 +846,18 @@ int enqueue_run(sddmm_ctx *c) {
             break;
         case SDDMM_EXACT:
             if (c->dtype == SDDMM_BF16)
-                hipLaunchKernelGGL(k_exact<DT_BF16>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                SDDMM_LAUNCH(c, k_exact<DT_BF16>, grid_for(c->nnz, BLOCK), BLOCK, c->dA,
                                    c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
             else if (c->dtype == SDDMM_F16)
-                hipLaunchKernelGGL(k_exact<DT_F16>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                SDDMM_LAUNCH(c, k_exact<DT_F16>, grid_for(c->nnz, BLOCK), BLOCK, c->dA,
                                    c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
             else
-                hipLaunchKernelGGL(k_exact<DT_F32>, dim3(grid_for(c->nnz, BLOCK)), dim3(BLOCK), 0, c->stream, c->dA,
+                SDDMM_LAUNCH(c, k_exact<DT_F32>, grid_for(c->nnz, BLOCK), BLOCK, c->dA,
                                    c->dB, c->K, c->d_rowidx, c->d_col, c->d_sval, c->dP, c->nnz);
             break;
         default: return fail(c, SDDMM_ERR_STATE, "no kernel for strategy %d", c->strategy);
     }
-    HIP_TRY(c, hipGetLastError());
+    LAUNCH_CHECK(c);
     c->stats.kernels_launched = c->launches;
     return SDDMM_OK;
 }
@@ -1141,10 +1169,10 @@ static int set_coo_common(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t
         }
         HIP_TRY(c, hipMemsetAsync(c->dP, 0, (size_t)nnz * sizeof(float), c->stream));
         const int g = grid_capped(nnz, 256);
-        hipLaunchKernelGGL(k_check_index, dim3(g), dim3(256), 0, c->stream, c->d_rowidx, nnz, M, c->d_pc);
-        hipLaunchKernelGGL(k_check_index, dim3(g), dim3(256), 0, c->stream, c->d_col, nnz, N, c->d_pc);
-        hipLaunchKernelGGL(k_check_coo_sorted, dim3(g), dim3(256), 0, c->stream, c->d_rowidx, nnz, c->d_pc);
-        HIP_TRY(c, hipGetLastError());
+        SDDMM_LAUNCH(c, k_check_index, g, 256, c->d_rowidx, nnz, M, c->d_pc);
+        SDDMM_LAUNCH(c, k_check_index, g, 256, c->d_col, nnz, N, c->d_pc);
+        SDDMM_LAUNCH(c, k_check_coo_sorted, g, 256, c->d_rowidx, nnz, c->d_pc);
+        LAUNCH_CHECK(c);
     }
     rc = fetch_counters(c);
     if (rc) { release_sparse(c); return rc; }
@@ -1154,14 +1182,14 @@ static int set_coo_common(sddmm_ctx *c, int M, int N, int64_t nnz, const int32_t
     }
     const bool sorted = c->pc.coo_unsorted == 0;
     if (sorted) {
-        hipLaunchKernelGGL(k_rowptr_from_sorted_coo, dim3(grid_for(nnz + 1, 256)), dim3(256), 0, c->stream,
+        SDDMM_LAUNCH(c, k_rowptr_from_sorted_coo, grid_for(nnz + 1, 256), 256,
                            c->d_rowidx, nnz, M, c->d_rowptr);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
         HIP_TRY(c, hipMemsetAsync(c->d_pc, 0, sizeof(DevCounters), c->stream));
         if (M > 0)
-            hipLaunchKernelGGL(k_check_rowptr, dim3(grid_for(M, 256)), dim3(256), 0, c->stream, c->d_rowptr, M, nnz,
+            SDDMM_LAUNCH(c, k_check_rowptr, grid_for(M, 256), 256, c->d_rowptr, M, nnz,
                                c->d_pc);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
         rc = fetch_counters(c);
         if (rc) { release_sparse(c); return rc; }
         if (c->pc.bad_pattern) {
@@ -1281,11 +1309,11 @@ static int plan_fused_items(sddmm_ctx *c) {
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     c->n_fused_items = 0;
     if (nb > 0) {
-        hipLaunchKernelGGL(k_classify_count, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+        SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr,
                            (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc);
-        hipLaunchKernelGGL(k_scan_block_sums, dim3(1), dim3(SCAN_BLOCK), 0, c->stream, c->d_block_sums, (int)nb,
+        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
         DevCounters tmp;
         HIP_TRY(c, hipMemcpyAsync(&tmp, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
         HIP_TRY(c, hipStreamSynchronize(c->stream));
@@ -1296,9 +1324,9 @@ static int plan_fused_items(sddmm_ctx *c) {
             c->fused_items_cap = c->n_fused_items;
         }
         if (c->n_fused_items > 0) {
-            hipLaunchKernelGGL(k_classify_write, dim3((unsigned)nb), dim3(SCAN_BLOCK), 0, c->stream, c->d_rowptr,
+            SDDMM_LAUNCH(c, k_classify_write, nb, SCAN_BLOCK, c->d_rowptr,
                                (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_fused_items);
-            HIP_TRY(c, hipGetLastError());
+            LAUNCH_CHECK(c);
         }
     }
     c->fused_items_valid = true;
@@ -1333,13 +1361,13 @@ int sddmm_run_fused(sddmm_ctx *c) {
                 const int64_t rows_per_wave = WAVE / LT::LPN;
                 const int64_t waves = ((int64_t)c->sM + rows_per_wave - 1) / rows_per_wave;
                 const int64_t rblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-                hipLaunchKernelGGL((k_fusedmm_rows<LT>), dim3((unsigned)xcd_grid(rblocks)), dim3(BLOCK), 0, c->stream,
+                SDDMM_LAUNCH(c, (k_fusedmm_rows<LT>), xcd_grid(rblocks), BLOCK,
                                    (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
                                    c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks);
                 ++launches;
                 if (c->n_fused_items > 0) {
                     const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-                    hipLaunchKernelGGL((k_fusedmm<LT>), dim3((unsigned)xcd_grid(nblocks)), dim3(BLOCK), 0, c->stream,
+                    SDDMM_LAUNCH(c, (k_fusedmm<LT>), xcd_grid(nblocks), BLOCK,
                                        (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col,
                                        c->d_sval, c->dP, c->dO, (const RowItem *)c->d_fused_items, c->n_fused_items,
                                        nblocks);
@@ -1347,7 +1375,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
                 }
             }
         });
-        HIP_TRY(c, hipGetLastError());
+        LAUNCH_CHECK(c);
     }
     HIP_TRY(c, hipEventRecord(c->ev1, c->stream));
     HIP_TRY(c, hipEventSynchronize(c->ev1));

@@ -59,9 +59,10 @@ def test_device_resident_operands(engine_factory):
         d_rp, d_col, d_val = hip.upload(rowptr), hip.upload(col), hip.upload(val)
         L = e.L
         e._chk(L.sddmm_set_dense_device(e.h, M, N, K, dA, dB, capi.F32))
-        e._chk(L.sddmm_set_csr_device(e.h, M, N, len(col), d_rp, d_col, d_val))
         e.nnz = len(col)
         for strategy in (capi.AUTO, capi.ROW_WAVE, capi.FLAT, capi.EXACT, capi.MFMA_TILE):
+            # set again for every strategy: that clears P, so no kernel can pass on the values of the one before
+            e._chk(L.sddmm_set_csr_device(e.h, M, N, len(col), d_rp, d_col, d_val))
             e.plan(strategy)
             e.run()
             got = e.values()
@@ -105,9 +106,9 @@ def test_device_resident_coo(engine_factory):
         L = e.L
         e.set_dense(A, B)
         d_r, d_c, d_v = hip.upload(r), hip.upload(c), hip.upload(v)
-        e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r, d_c, d_v))
         e.nnz = len(r)
         for strategy in (capi.AUTO, capi.ROW_WAVE, capi.FLAT, capi.MFMA_TILE, capi.EXACT):
+            e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r, d_c, d_v))     # clears P
             e.plan(strategy)
             e.run()
             assert O.check_values(e.values(), ref, mag=mag)[0], capi.STRATEGY_NAMES[strategy]
@@ -115,8 +116,8 @@ def test_device_resident_coo(engine_factory):
             e.update_values(v)                       # borrowed values
         perm = rng.permutation(len(r))
         d_r2, d_c2, d_v2 = hip.upload(r[perm]), hip.upload(c[perm]), hip.upload(v[perm])
-        e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r2, d_c2, d_v2))
         for strategy in (capi.AUTO, capi.FLAT, capi.EXACT):
+            e._chk(L.sddmm_set_coo_device(e.h, M, N, len(r), d_r2, d_c2, d_v2))
             e.plan(strategy)
             e.run()
             got = e.values()
@@ -158,8 +159,8 @@ def test_operand_beyond_4gib_uses_64bit_offsets(engine_factory):
     assert np.count_nonzero(ref) > 0.9 * len(ref)
     e = engine_factory()
     e.set_dense(A, B)
-    e.set_csr(M, N, rowptr, col, val)
     for strategy in (capi.AUTO, capi.FLAT, capi.ROW_WAVE, capi.SHORT_ROWS, capi.LDS_TILED, capi.MFMA_TILE, capi.EXACT):
+        e.set_csr(M, N, rowptr, col, val)            # clears P
         e.plan(strategy)
         e.run()
         got = e.values()

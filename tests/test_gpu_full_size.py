@@ -46,7 +46,9 @@ def test_full_size(engine_factory, name, K, other):
     e.run()
     np.testing.assert_array_equal(e.values(), auto * f32(2))
     e.update_values(w.sval)
-    # a fixed strategy on the same context
+    # a fixed strategy on the same context (the pattern is set again: that clears P, so a
+    # kernel that wrote nothing could not pass on the previous strategy's values)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
     e.plan(other)
     e.run()
     fixed = e.values()
@@ -54,6 +56,7 @@ def test_full_size(engine_factory, name, K, other):
     if st.mfma_tiles == 0 and st.panels == 0:        # only gather kernels: same per-entry arithmetic
         np.testing.assert_array_equal(fixed.view(np.uint32), auto.view(np.uint32))
     # the exact-order kernel is the CPU loop bit for bit, also at this size
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
     e.plan(capi.EXACT)
     e.run()
     np.testing.assert_array_equal(e.values().view(np.uint32), ref.view(np.uint32))
@@ -82,10 +85,10 @@ def test_positions_beyond_2_to_the_30(engine_factory):
         A[sample // L].astype(np.float64) * B[col[sample]].astype(np.float64)).sum(axis=1)
     e = engine_factory()
     e.set_dense(A, B)
-    e.set_csr(M, N, rowptr, col, val)
     step = 1 << 26
     for strategy in (capi.EXACT, capi.AUTO, capi.FLAT):
         print("strategy", capi.STRATEGY_NAMES[strategy], flush=True)
+        e.set_csr(M, N, rowptr, col, val)                  # clears P
         e.plan(strategy)
         e.run()
         got = e.values()
@@ -104,3 +107,36 @@ def test_positions_beyond_2_to_the_30(engine_factory):
         assert ok, (capi.STRATEGY_NAMES[strategy], int(sample[j]), worst)
         del got
     e.close()
+
+
+def test_a_grid_beyond_one_dispatch_is_refused_not_truncated(engine_factory):
+    """2^26 + 1000 rows: one wavefront per row would be a launch of more than 2^32 threads,
+    of which the hardware would run a part without any error.  The library must refuse that
+    strategy and compute the same matrix with the strategies that fit."""
+    M, N, K = (1 << 26) + 1000, 64, 4
+    rng = np.random.default_rng(8)
+    rowptr = np.arange(M + 1, dtype=np.int32)              # one entry per row
+    col = rng.integers(0, N, M).astype(np.int32)
+    val = rng.random(M, dtype=f32)
+    A = rng.random((M, K), dtype=f32)
+    B = rng.random((N, K), dtype=f32)
+    ref = O.sddmm_csr(rowptr, col, val, A, B, threads=0)
+    for strategy in (capi.ROW_WAVE, capi.AUTO, capi.FLAT, capi.EXACT):
+        print("strategy", capi.STRATEGY_NAMES[strategy], flush=True)
+        e = engine_factory()                               # a fresh context: P starts at zero
+        e.set_dense(A, B)
+        e.set_csr(M, N, rowptr, col, val)
+        if strategy == capi.ROW_WAVE:
+            e.plan(strategy)
+            with pytest.raises(capi.SddmmError) as ei:
+                e.run()
+            assert ei.value.code == capi.ERR_UNSUPPORTED and "2^32" in str(ei.value)
+        else:
+            e.plan(strategy)
+            e.run()
+            got = e.values()
+            if strategy == capi.EXACT:
+                assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+            else:
+                assert float(np.abs(got - ref).max()) <= 1e-5 * K      # |ref| < K
+        e.close()

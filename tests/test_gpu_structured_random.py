@@ -69,8 +69,8 @@ def test_structured_random(engine_factory, seed):
     _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
     e = engine_factory()
     e.set_dense(A, B)
-    e.set_csr(M, N, rowptr, col, val)
     for strategy in STRATEGIES:
+        e.set_csr(M, N, rowptr, col, val)    # again for every strategy: clears P, nothing passes on stale values
         e.plan(strategy)
         e.run()
         got = e.values()
@@ -88,6 +88,7 @@ def test_structured_random(engine_factory, seed):
         _, magb = O.sddmm_csr_f64(rowptr, col, val, Af, Bf)
         e.set_dense(Ab, Bb, capi.BF16)
         for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED):
+            e.set_csr(M, N, rowptr, col, val)
             e.plan(strategy)
             e.run()
             ok, worst, i = O.check_values(e.values(), refb, mag=magb)
@@ -167,8 +168,8 @@ def test_strip_classifier_matches_host_model(engine_factory, monkeypatch, seed):
     _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
     e = engine_factory()
     e.set_dense(A, B)
-    e.set_csr(M, N, rowptr, col, val)
     for strategy, min_fill in ((capi.MFMA_TILE, 1), (capi.AUTO, 96)):
+        e.set_csr(M, N, rowptr, col, val)    # clears P
         e.plan(strategy)
         e.run()
         st = e.stats()
@@ -183,6 +184,7 @@ def test_strip_classifier_matches_host_model(engine_factory, monkeypatch, seed):
     # still has exactly one owner
     natural = (st.mfma_tiles, st.nnz_mfma) if st.strategy_used != capi.FLAT else (0, 0)
     monkeypatch.setenv("SDDMM_GATHERED", "1")
+    e.set_csr(M, N, rowptr, col, val)
     e.plan(capi.AUTO)
     e.run()
     st = e.stats()
@@ -263,10 +265,10 @@ def test_similarity_mixtures(engine_factory, seed):
         e.set_dense(Ab, Bb, capi.F16)
     else:
         e.set_dense(A, B)
-    e.set_csr(M, N, rowptr, col, val)
     ref = O.sddmm_csr(rowptr, col, val, A, B)
     _, mag = O.sddmm_csr_f64(rowptr, col, val, A, B)
     for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED, capi.FLAT):
+        e.set_csr(M, N, rowptr, col, val)    # clears P
         e.plan(strategy)
         e.run()
         st = e.stats()
