@@ -285,6 +285,33 @@ def test_context_reuse_and_update_values(engine_factory):
     e.close()
 
 
+@pytest.mark.parametrize("name", ["fem_banded", "mixed_density", "similar_rows"])
+def test_non_finite_operands_stay_in_their_own_entries(engine_factory, name):
+    """A NaN in one B row and an infinity in one A row: exactly the entries that involve
+    them are non-finite, as in the CPU loop; the matrix-core paths compute whole tiles and
+    panels, and nothing of a poisoned row or column may leak into its neighbours."""
+    w = W.make(name, "small", K=32)
+    A, B = w.A.copy(), w.B.copy()
+    rows_of = np.repeat(np.arange(w.M), np.diff(w.rowptr))
+    bad_col = int(w.col[len(w.col) // 2])
+    bad_row = int(rows_of[len(w.col) // 3])
+    B[bad_col, 5] = np.nan
+    A[bad_row, 7] = np.inf
+    with np.errstate(all="ignore"):
+        ref = O.sddmm_csr(w.rowptr, w.col, w.sval, A, B, threads=0)
+    poisoned = (w.col == bad_col) | (rows_of == bad_row)
+    assert poisoned.any() and np.array_equal(~np.isfinite(ref), poisoned)
+    clean = ~poisoned
+    _, mag = O.sddmm_csr_f64(w.rowptr[:], w.col, np.where(clean, w.sval, 0).astype(f32), w.A, w.B)
+    for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED, capi.FLAT, capi.ROW_WAVE):
+        got, st = run_csr(engine_factory, w.rowptr, w.col, w.sval, A, B, w.N, strategy)
+        what = "%s %s" % (name, capi.STRATEGY_NAMES[strategy])
+        assert np.array_equal(~np.isfinite(got), poisoned), what
+        assert np.array_equal(np.isnan(got), np.isnan(ref)), what
+        ok, worst, i = O.check_values(got[clean], ref[clean], mag=mag[clean])
+        assert ok, (what, i, worst)
+
+
 def test_replaced_operands_are_planned_again_as_last_asked(engine_factory):
     rng = np.random.default_rng(14)
     e = engine_factory()
