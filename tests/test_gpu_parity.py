@@ -312,6 +312,25 @@ def test_non_finite_operands_stay_in_their_own_entries(engine_factory, name):
         assert ok, (what, i, worst)
 
 
+@pytest.mark.parametrize("name", ["fem_banded", "mixed_density"])
+def test_denormal_results_are_not_flushed(engine_factory, name):
+    """Operands of magnitude 1e-20: every product and every result is a denormal fp32
+    number.  The CPU loop keeps them; so must the vector and the matrix-core paths.
+    Sums of denormals are exact, so the only differences allowed are the roundings of
+    the K products (one step of 2^-149 each, fused or not)."""
+    K = 32
+    w = W.make(name, "small", K=K)
+    A = (w.A * f32(1e-20)).astype(f32)
+    B = (w.B * f32(1e-20)).astype(f32)
+    ref = O.sddmm_csr(w.rowptr, w.col, w.sval, A, B, threads=0)
+    assert 0 < float(np.abs(ref).max()) < 1.17e-38 and np.count_nonzero(ref) > 0.99 * len(ref)
+    for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED, capi.FLAT, capi.EXACT):
+        got, _ = run_csr(engine_factory, w.rowptr, w.col, w.sval, A, B, w.N, strategy)
+        what = "%s %s" % (name, capi.STRATEGY_NAMES[strategy])
+        assert np.count_nonzero(got) >= np.count_nonzero(ref) - 5, what
+        assert float(np.abs(got.astype(np.float64) - ref).max()) <= (K + 1) * 2.0 ** -149, what
+
+
 def test_replaced_operands_are_planned_again_as_last_asked(engine_factory):
     rng = np.random.default_rng(14)
     e = engine_factory()
