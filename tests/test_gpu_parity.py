@@ -110,7 +110,7 @@ def test_random_matrices_like_the_reference_tests(engine_factory, case, strategy
 
 # every K from 1 up, powers of two, multiples of 4 that are not powers of two,
 # odd K (scalar pieces) and K beyond one piece per lane
-KS = [1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 31, 32, 33, 48, 64, 96, 100, 128, 160, 256, 260, 300, 512, 1024]
+KS = [1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 31, 32, 33, 48, 64, 96, 100, 128, 160, 256, 260, 300, 512, 1024, 2048, 4097]
 
 
 @pytest.mark.parametrize("K", KS)
