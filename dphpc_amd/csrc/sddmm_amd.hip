@@ -1061,6 +1061,9 @@ static int set_dense_common(sddmm_ctx *c, int M, int N, int K, const void *A, co
         return fail(c, SDDMM_ERR_INVALID, "unknown dtype %d", dtype);
     if (dtype != SDDMM_F32 && K % 8) return fail(c, SDDMM_ERR_INVALID, "16-bit operands need K %% 8 == 0 (got %d)", K);
     if ((M > 0 && !A) || (N > 0 && !B)) return fail(c, SDDMM_ERR_NULL, "A or B is NULL");
+    // a plan depends on the pattern and on the shape and type of the dense operands, not on their
+    // values: new A and B of the same shape (the next iteration of a solver) keep it
+    const bool keep_plan = c->planned && c->have_dense && c->M == M && c->N == N && c->K == K && c->dtype == dtype;
     release_dense(c);
     const size_t es = elem_size(dtype);
     const size_t a_bytes = (size_t)M * K * es, b_bytes = (size_t)N * K * es;
@@ -1079,7 +1082,7 @@ static int set_dense_common(sddmm_ctx *c, int M, int N, int K, const void *A, co
     }
     c->M = M; c->N = N; c->K = K; c->dtype = dtype;
     c->have_dense = true;
-    c->planned = false;
+    c->planned = keep_plan;
     return SDDMM_OK;
 }
 

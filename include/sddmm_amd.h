@@ -159,9 +159,11 @@ int sddmm_update_values(sddmm_ctx *ctx, const float *sval);
 
 /* ---- plan (init phase) + run -------------------------------------------- */
 /* Classify rows / tiles and build whatever the chosen strategy needs.  All of it
- * runs on the device; nothing is read back except a few counters.  Replacing an
- * operand (sddmm_set_*) drops the plan; the next run then plans again by itself with
- * the strategy asked for last (SDDMM_AUTO on a context that was never planned). */
+ * runs on the device; nothing is read back except a few counters.  Replacing the
+ * sparse operand, or the dense ones by operands of another shape or type, drops the
+ * plan; the next run then plans again by itself with the strategy asked for last
+ * (SDDMM_AUTO on a context that was never planned).  New A and B of the same shape and
+ * type keep the plan: it depends on the pattern only. */
 int sddmm_plan(sddmm_ctx *ctx, int strategy);
 /* Launch and wait.  P is complete on return (every reference run_csr ends in a
  * device synchronise, e.g. src/competitors/gpu/gpu_basic.hpp:72). */

@@ -353,6 +353,33 @@ def test_replaced_operands_are_planned_again_as_last_asked(engine_factory):
     e.close()
 
 
+def test_new_dense_values_of_the_same_shape_keep_the_plan(engine_factory):
+    # iterations of a solver: the same S, new A and B every time
+    rng = np.random.default_rng(15)
+    w = W.make("mixed_density", "small", K=32)
+    e = engine_factory()
+    e.set_dense(w.A, w.B)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    e.plan(capi.AUTO)
+    planned = e.stats().plan_ms
+    assert planned > 0
+    for it in range(3):
+        A = rng.uniform(-1, 1, w.A.shape).astype(f32)
+        B = rng.uniform(-1, 1, w.B.shape).astype(f32)
+        e.set_dense(A, B)
+        e.run()
+        assert e.stats().plan_ms == planned                    # no new plan was made
+        assert_parity(e.values(), w.rowptr, w.col, w.sval, A, B, what="iteration %d" % it)
+    # another width is another plan
+    A = rng.uniform(-1, 1, (w.M, 64)).astype(f32)
+    B = rng.uniform(-1, 1, (w.N, 64)).astype(f32)
+    e.set_dense(A, B)
+    e.run()
+    assert e.stats().plan_ms != planned
+    assert_parity(e.values(), w.rowptr, w.col, w.sval, A, B, what="K=64")
+    e.close()
+
+
 def test_distinct_contexts_on_distinct_threads(engine_factory):
     """A context is single-threaded, but two contexts driven from two host threads at
     once (each on its own stream) must not disturb each other: every result of every
