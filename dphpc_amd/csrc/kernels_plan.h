@@ -268,6 +268,33 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_block_sums(unsigned int *__
     if (threadIdx.x == 0) *total_out = carry;
 }
 
+// the whole exclusive scan of a short array in one workgroup (one launch instead of three)
+constexpr int SCAN_SMALL_ITEMS = 8;
+constexpr int SCAN_SMALL_MAX = 16384;
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_small(const unsigned int *__restrict__ in, int n,
+                                                           unsigned int *__restrict__ out,
+                                                           unsigned long long *__restrict__ total_out) {
+    unsigned int carry = 0;
+    for (int base = 0; base < n; base += SCAN_BLOCK * SCAN_SMALL_ITEMS) {
+        const int i0 = base + (int)threadIdx.x * SCAN_SMALL_ITEMS;
+        unsigned int v[SCAN_SMALL_ITEMS], mine = 0;
+#pragma unroll
+        for (int q = 0; q < SCAN_SMALL_ITEMS; ++q) {
+            v[q] = i0 + q < n ? in[i0 + q] : 0u;
+            mine += v[q];
+        }
+        unsigned int total;
+        unsigned int at = carry + block_exclusive_scan(mine, &total);
+#pragma unroll
+        for (int q = 0; q < SCAN_SMALL_ITEMS; ++q) {
+            if (i0 + q < n) out[i0 + q] = at;
+            at += v[q];
+        }
+        carry += total;
+    }
+    if (threadIdx.x == 0) *total_out = carry;
+}
+
 // pass 3: write the items
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__restrict__ rowptr,
                                                                const unsigned char *__restrict__ owner, int M,

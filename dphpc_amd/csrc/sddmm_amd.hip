@@ -445,6 +445,11 @@ int classify_rows(sddmm_ctx *c) {
 
 // Exclusive scan of n unsigned ints on the device (in != out), total to *d_total.
 int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t n, unsigned long long *d_total) {
+    if (n <= SCAN_SMALL_MAX) {
+        SDDMM_LAUNCH(c, k_scan_small, 1, SCAN_BLOCK, in, (int)n, out, d_total);
+        LAUNCH_CHECK(c);
+        return SDDMM_OK;
+    }
     const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
     if (nb > c->block_sums_cap) {
         dfree(c->d_block_sums);
