@@ -404,7 +404,9 @@ void launch_auto(sddmm_ctx *c) {
 }
 
 // Row classifier: statistics, then the item list of the wave-per-segment kernel.
-int classify_rows(sddmm_ctx *c) {
+// Row classes and work items of the rows nobody owns, in two halves around a read-back of the
+// counters: the count (launch only; it may be launched again after more rows found an owner) ...
+int classify_rows_count(sddmm_ctx *c) {
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     if (nb > c->block_sums_cap) {
         dfree(c->d_block_sums);
@@ -423,8 +425,11 @@ int classify_rows(sddmm_ctx *c) {
                            &c->d_pc->n_items);
         LAUNCH_CHECK(c);
     }
-    int rc = fetch_counters(c);
-    if (rc) return rc;
+    return SDDMM_OK;
+}
+// ... and the items, once the counters are on the host (nothing may use the block sums in between)
+int classify_rows_items(sddmm_ctx *c) {
+    const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     c->n_items = (int64_t)c->pc.n_items;
     c->rows_short = (int64_t)c->pc.rows_short;
     c->rpw = env_int("SDDMM_RPW", rows_per_wave(c->rows_short ? (double)c->pc.nnz_short / (double)c->rows_short : 0.0));
@@ -572,7 +577,8 @@ int plan_gathered_candidates(sddmm_ctx *c, int min_len) {
 }
 
 // after the fetch_counters that follows plan_gathered_candidates
-int plan_gathered_count(sddmm_ctx *c, int min_fill) {
+int plan_gathered_count(sddmm_ctx *c, int min_fill, bool *launched) {
+    *launched = false;
     if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
     c->n_cand = (int64_t)c->raw.n_candidates;
     if (c->n_cand < 2) { c->n_cand = 0; return SDDMM_OK; }
@@ -602,8 +608,11 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill) {
     LAUNCH_CHECK(c);
     rc = device_scan(c, c->d_vstrip_ntiles, c->d_vstrip_off, c->n_vstrips, &c->d_pc->tiles_scanned);
     if (rc) return rc;
-    rc = fetch_counters(c);
-    if (rc) return rc;
+    *launched = true;
+    return SDDMM_OK;
+}
+// after the counters came back
+int plan_gathered_take(sddmm_ctx *c) {
     c->n_tiles = (int64_t)c->pc.n_tiles + c->n_tiles_union;
     c->nnz_tiles = (int64_t)c->pc.nnz_tiles + c->nnz_tiles_union;
     if ((int64_t)c->pc.tiles_scanned != (int64_t)c->pc.n_tiles - c->n_tiles_natural)
@@ -913,6 +922,12 @@ int do_plan(sddmm_ctx *c, int strategy) {
                 rc = plan_gathered_candidates(c, std::max(16, env_int("SDDMM_GATHERED_MIN", 64)));
                 if (rc) return rc;
             }
+            // the rows nobody owns so far are classified in the same batch: most matrices have
+            // no gathered strips, and their plan then waits for the device once
+            c->ts = std::max(1, env_int("SDDMM_TS", 24));
+            c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+            rc = classify_rows_count(c);
+            if (rc) return rc;
             rc = fetch_counters(c);
             if (rc) return rc;
             rc = take_tile_counts(c);
@@ -920,16 +935,24 @@ int do_plan(sddmm_ctx *c, int strategy) {
             rc = plan_panels_items(c, pseg);
             if (rc) return rc;
             if (gathered) {
-                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)));
+                bool launched = false;
+                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)), &launched);
                 if (rc) return rc;
+                if (launched) {
+                    // gathered strips may have taken rows: classify again, one more read-back
+                    rc = classify_rows_count(c);
+                    if (rc) return rc;
+                    rc = fetch_counters(c);
+                    if (rc) return rc;
+                    rc = plan_gathered_take(c);
+                    if (rc) return rc;
+                }
             }
             if (resolved != SDDMM_LDS_TILED) {
                 rc = plan_tiles_fill(c);
                 if (rc) return rc;
             }
-            c->ts = std::max(1, env_int("SDDMM_TS", 24));
-            c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
-            rc = classify_rows(c);
+            rc = classify_rows_items(c);
             if (rc) return rc;
             // A matrix whose rows are short on average (fewer than 32 entries per non-empty
             // row), with no strip or panel taken, is a flat stream of entries: the flat
