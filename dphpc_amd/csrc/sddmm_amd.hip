@@ -55,6 +55,7 @@ struct sddmm_ctx {
     int requested = SDDMM_AUTO;
     DevCounters *d_pc = nullptr;     // device counters
     DevCounters raw{};               // host copy of the device block
+    DevCounters *h_pc = nullptr;     // pinned landing place of the read-back (no staging copy)
     PlanCounters pc{};               // its summary
     sddmm_stats stats{};
     // AUTO: rows shorter than ts go to the many-rows-per-wave kernel, the others
@@ -224,8 +225,9 @@ int grid_capped(int64_t n, int block, int cap = 16384) {
 }
 
 int fetch_counters(sddmm_ctx *c) {
-    HIP_TRY(c, hipMemcpyAsync(&c->raw, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(c, hipMemcpyAsync(c->h_pc, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(c, hipStreamSynchronize(c->stream));
+    c->raw = *c->h_pc;
     c->pc = summarize(c->raw);
     return SDDMM_OK;
 }
@@ -1041,7 +1043,8 @@ int sddmm_create(sddmm_ctx **out, int device) {
     if (!c) return SDDMM_ERR_ALLOC;
     c->device = device;
     if (hipStreamCreate(&c->own_stream) != hipSuccess || hipEventCreate(&c->ev0) != hipSuccess ||
-        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(DevCounters)) != hipSuccess) {
+        hipEventCreate(&c->ev1) != hipSuccess || hipMalloc((void **)&c->d_pc, sizeof(DevCounters)) != hipSuccess ||
+        hipHostMalloc((void **)&c->h_pc, sizeof(DevCounters), hipHostMallocDefault) != hipSuccess) {
         sddmm_destroy(c);
         return SDDMM_ERR_HIP;
     }
@@ -1074,6 +1077,7 @@ void sddmm_destroy(sddmm_ctx *c) {
     release_sparse(c);
     dfree(c->dO);
     dfree(c->d_pc);
+    if (c->h_pc) (void)hipHostFree(c->h_pc);
     if (c->ev0) (void)hipEventDestroy(c->ev0);
     if (c->ev1) (void)hipEventDestroy(c->ev1);
     if (c->own_stream) (void)hipStreamDestroy(c->own_stream);
