@@ -44,37 +44,5 @@ def build_library(verbose=False, extra_flags=(), out=None):
     return LIB_PATH
 
 
-PROBE_PATH = os.path.join(LIB_DIR, "copy_probe")
-
-
-def build_copy_probe(verbose=False):
-    """Stand-alone plain copy kernel used to calibrate rocprofv3's byte counters."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-o", PROBE_PATH, os.path.join(CSRC, "copy_probe.hip")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
-    return PROBE_PATH
-
-
-GATHER_PROBE_PATH = os.path.join(LIB_DIR, "gather_probe")
-
-
-def build_gather_probe(verbose=False):
-    """Stand-alone row-gather kernel: the ceiling of the box for 128-byte row gathers."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-o", GATHER_PROBE_PATH, os.path.join(CSRC, "gather_probe.hip")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
-    return GATHER_PROBE_PATH
-
-
 if __name__ == "__main__":
     print(build_library(verbose=True))
-    print(build_copy_probe(verbose=True))
-    print(build_gather_probe(verbose=True))

@@ -84,13 +84,17 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
                     const float d = U::dot(a.u[i], bf[q][i], p);
                     p = C::unit_on(j, i, KU) ? d : p;
                 }
-                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);
+                // a step past the end of the row works on a clamped position: it must leave the
+                // output row alone whatever that position's B row holds (0 * inf is not 0)
+                const bool live = __shfl((int)valid, src, WAVE) != 0;
+                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);     // every lane takes part in the lane exchange
+                p = live ? p : 0.f;
 #pragma unroll
                 for (int i = 0; i < UPL; ++i) {
-                    acc[i].x = __builtin_fmaf(p, bf[q][i].x, acc[i].x);
-                    acc[i].y = __builtin_fmaf(p, bf[q][i].y, acc[i].y);
-                    acc[i].z = __builtin_fmaf(p, bf[q][i].z, acc[i].z);
-                    acc[i].w = __builtin_fmaf(p, bf[q][i].w, acc[i].w);
+                    acc[i].x = live ? __builtin_fmaf(p, bf[q][i].x, acc[i].x) : acc[i].x;
+                    acc[i].y = live ? __builtin_fmaf(p, bf[q][i].y, acc[i].y) : acc[i].y;
+                    acc[i].z = live ? __builtin_fmaf(p, bf[q][i].z, acc[i].z) : acc[i].z;
+                    acc[i].w = live ? __builtin_fmaf(p, bf[q][i].w, acc[i].w) : acc[i].w;
                 }
                 if (j == t0 + q) out = p;
             }
@@ -204,13 +208,17 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
                     const float d = U::dot(a.u[i], bf[q][i], p);
                     p = C::unit_on(j, i, KU) ? d : p;
                 }
-                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);
+                // a step past the end of the row works on a clamped position: it must leave the
+                // output row alone whatever that position's B row holds (0 * inf is not 0)
+                const bool live = __shfl((int)has, src, WAVE) != 0;
+                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);     // every lane takes part in the lane exchange
+                p = live ? p : 0.f;
 #pragma unroll
                 for (int i = 0; i < UPL; ++i) {
-                    acc[i].x = __builtin_fmaf(p, bf[q][i].x, acc[i].x);
-                    acc[i].y = __builtin_fmaf(p, bf[q][i].y, acc[i].y);
-                    acc[i].z = __builtin_fmaf(p, bf[q][i].z, acc[i].z);
-                    acc[i].w = __builtin_fmaf(p, bf[q][i].w, acc[i].w);
+                    acc[i].x = live ? __builtin_fmaf(p, bf[q][i].x, acc[i].x) : acc[i].x;
+                    acc[i].y = live ? __builtin_fmaf(p, bf[q][i].y, acc[i].y) : acc[i].y;
+                    acc[i].z = live ? __builtin_fmaf(p, bf[q][i].z, acc[i].z) : acc[i].z;
+                    acc[i].w = live ? __builtin_fmaf(p, bf[q][i].w, acc[i].w) : acc[i].w;
                 }
                 if (j == q0 + q) out = p;
             }

@@ -879,6 +879,9 @@ int enqueue_run(sddmm_ctx *c) {
 }
 
 int do_plan(sddmm_ctx *c, int strategy) {
+    // the plan state is rewritten in place: a plan that fails half way must not leave the
+    // previous one looking valid (its items exclude rows that tiles and panels owned)
+    c->planned = false;
     int resolved = strategy;
     const bool csr_ok = c->have_rowptr;
     // without a row pointer (unsorted COO) only the flat kernels apply

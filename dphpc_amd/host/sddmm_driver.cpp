@@ -12,13 +12,14 @@
 //   correctness,num_thread_blocks,num_threads_per_block
 // init/cleanup/total are host wall-clock like the reference's; comp_ns is the
 // device time of run_* from HIP events recorded by the library on its launch
-// stream.  The correctness baseline is competitors[0] as in the reference
-// (benchmark.hpp:50-61); here that is GPU-AMD-Exact, the kernel that repeats the
-// CPU loop's operation order.  A run counts as correct when the pattern is
-// identical and every value is within 1e-5 * max(|expected|, 0.25 * mag) where
-// mag = |S| * sum_k |a_k b_k| is obtained from one more SDDMM on the absolute
-// values of the operands: with signed inputs some entries cancel almost to zero
-// and a purely relative test (the reference's, CSR.hpp:92-94) is meaningless there.
+// stream for the GPU competitors, host wall-clock for CPU-Basic.  The correctness
+// baseline is competitors[0] as in the reference (benchmark.hpp:50-61, main.cpp:18-22):
+// CPU-Basic, the plain host loop (cpu_host.hpp), whose CSV rows come first.
+// GPU-AMD-Exact repeats the CPU loop's operation order and must match it bit for
+// bit; every other competitor counts as correct when the pattern is identical and
+// every value is within 1e-5 * max(|expected|, 0.25 * mag), mag = |S| * sum_k |a_k b_k|
+// computed on the host: with signed inputs some entries cancel almost to zero and a
+// purely relative test (the reference's, CSR.hpp:92-94) is meaningless there.
 #include <chrono>
 #include <cmath>
 #include <cstdio>
@@ -29,16 +30,18 @@
 #include <string>
 #include <vector>
 
+#include "cpu_host.hpp"
 #include "datasets.hpp"
 #include "gpu_amd.hpp"
 
 using Clock = std::chrono::high_resolution_clock;
 using sddmm_host::Dataset;
+using CompetitorPtr = std::shared_ptr<SDDMM::Competitor<float>>;
 
 struct Timing { long long total_ns, init_ns, comp_ns, cleanup_ns; };
 
 template <class F1, class F2, class F3>
-static Timing timed(Competitors::GPUAmd &c, F1 init, F2 run, F3 cleanup) {
+static Timing timed(SDDMM::Competitor<float> &c, F1 init, F2 run, F3 cleanup) {
     const auto t0 = Clock::now();
     init();
     const auto t1 = Clock::now();
@@ -48,47 +51,47 @@ static Timing timed(Competitors::GPUAmd &c, F1 init, F2 run, F3 cleanup) {
     const auto t3 = Clock::now();
     auto ns = [](auto a, auto b) { return (long long)std::chrono::duration_cast<std::chrono::nanoseconds>(b - a).count(); };
     Timing t{ns(t0, t3), ns(t0, t1), ns(t1, t2), ns(t2, t3)};
-    if (c.last_ok()) t.comp_ns = (long long)(c.last_stats().run_ms * 1e6);
+    // device time for the GPU competitors (the reference brackets run_* of an is_gpu()
+    // competitor with device events, benchmark.hpp:148-190)
+    if (auto *g = dynamic_cast<Competitors::GPUAmd *>(&c))
+        if (g->last_ok()) t.comp_ns = (long long)(g->last_stats().run_ms * 1e6);
     return t;
 }
 
-// |S| * sum_k |a_k * b_k| per stored entry, computed by the exact-order kernel
-static std::vector<float> magnitudes(Dataset &d) {
-    auto absd = [](Dense<float> &m) {
-        std::vector<float> flat(m.get_pointer(), m.get_pointer() + (size_t)m.getRows() * m.getCols());
-        for (auto &x : flat) x = std::fabs(x);
-        return Dense<float>(m.getRows(), m.getCols(), std::move(flat));
-    };
-    Dense<float> A = absd(d.A), B = absd(d.B);
-    CSR<float> S(d.S_csr);
-    for (auto &v : S.getValues()) v = std::fabs(v);
-    CSR<float> P(S);
-    P.clearValues();
-    Competitors::GPUAmd c(SDDMM_EXACT);
-    c.init_csr(A, B, S, P);
-    c.run_csr(A, B, S, P);
-    c.cleanup_csr(A, B, S, P);
-    return P.getValues();
+static bool ran_ok(SDDMM::Competitor<float> &c) {
+    auto *g = dynamic_cast<Competitors::GPUAmd *>(&c);
+    return g ? g->last_ok() : true;
 }
 
-static bool values_ok(const std::vector<float> &got, const std::vector<float> &exp, const std::vector<float> &mag) {
+static bool values_ok(const std::vector<float> &got, const std::vector<float> &exp, const std::vector<double> &mag,
+                      bool bitwise) {
     if (got.size() != exp.size() || got.size() != mag.size()) return false;
+    if (bitwise) return got.empty() || std::memcmp(got.data(), exp.data(), got.size() * sizeof(float)) == 0;
     for (size_t i = 0; i < got.size(); ++i) {
-        const double scale = std::max(std::fabs((double)exp[i]), 0.25 * (double)mag[i]);
+        const double scale = std::max(std::fabs((double)exp[i]), 0.25 * mag[i]);
         if (!(std::fabs((double)got[i] - (double)exp[i]) <= 1e-5 * scale)) return false;
     }
     return true;
 }
 
-static void bench_dataset(Dataset &d, std::vector<std::shared_ptr<Competitors::GPUAmd>> &comps, int num_runs) {
+static void bench_dataset(Dataset &d, std::vector<CompetitorPtr> &comps, int num_runs) {
+    // expected result: competitors[0] on the CSR form, before anything is timed
     CSR<float> expected_csr(d.S_csr);
-    COO<float> expected_coo(d.S_coo);
-    bool have_expected = false;
-    const std::vector<float> mag = magnitudes(d);
+    expected_csr.clearValues();
+    {
+        SDDMM::Competitor<float> &base = *comps[0];
+        base.init_csr(d.A, d.B, d.S_csr, expected_csr);
+        base.run_csr(d.A, d.B, d.S_csr, expected_csr);
+        base.cleanup_csr(d.A, d.B, d.S_csr, expected_csr);
+    }
+    COO<float> expected_coo(expected_csr);
+    const std::vector<double> mag = Competitors::CPUHost::magnitudes(d.A, d.B, d.S_csr);
     const int K = (int)d.A.getCols();
     for (auto &cp : comps) {
-        Competitors::GPUAmd &c = *cp;
+        SDDMM::Competitor<float> &c = *cp;
+        const bool bitwise = c.name == "CPU-Basic" || c.name == "GPU-AMD-Exact";
         for (int fmt = 0; fmt < 2; ++fmt) {
+            if (fmt == 0 ? !c.csr_supported() : !c.coo_supported()) continue;
             for (int run = 0; run < num_runs; ++run) {
                 Timing t;
                 bool correct;
@@ -97,18 +100,17 @@ static void bench_dataset(Dataset &d, std::vector<std::shared_ptr<Competitors::G
                     P.clearValues();
                     t = timed(c, [&] { c.init_csr(d.A, d.B, d.S_csr, P); }, [&] { c.run_csr(d.A, d.B, d.S_csr, P); },
                               [&] { c.cleanup_csr(d.A, d.B, d.S_csr, P); });
-                    if (!have_expected) { expected_csr = P; expected_coo = COO<float>(P); have_expected = c.last_ok(); }
-                    correct = c.last_ok() && P.getRowPositions() == expected_csr.getRowPositions() &&
+                    correct = ran_ok(c) && P.getRowPositions() == expected_csr.getRowPositions() &&
                               P.getColPositions() == expected_csr.getColPositions() &&
-                              values_ok(P.getValues(), expected_csr.getValues(), mag);
+                              values_ok(P.getValues(), expected_csr.getValues(), mag, bitwise);
                 } else {
                     COO<float> P(d.S_coo);
                     P.clearValues();
                     t = timed(c, [&] { c.init_coo(d.A, d.B, d.S_coo, P); }, [&] { c.run_coo(d.A, d.B, d.S_coo, P); },
                               [&] { c.cleanup_coo(d.A, d.B, d.S_coo, P); });
-                    correct = c.last_ok() && P.getRowPositions() == expected_coo.getRowPositions() &&
+                    correct = ran_ok(c) && P.getRowPositions() == expected_coo.getRowPositions() &&
                               P.getColPositions() == expected_coo.getColPositions() &&
-                              values_ok(P.getValues(), expected_coo.getValues(), mag);
+                              values_ok(P.getValues(), expected_coo.getValues(), mag, bitwise);
                 }
                 std::cout << c.name << "," << d.name << "," << (fmt == 0 ? "CSR" : "COO") << "," << d.S_coo.getRows() << ","
                           << d.S_coo.getCols() << "," << K << "," << d.S_coo.getValues().size() << "," << t.total_ns << ","
@@ -137,7 +139,8 @@ int main(int argc, char **argv) {
         else { std::fprintf(stderr, "usage: %s [--K k] [--num_runs n] [--scale s] [--dataset name|file.mtx|edges.txt] [--dim n] [--no_csv_header]\n", argv[0]); return 2; }
     }
     if (K < 1 || num_runs < 1 || scale <= 0) { std::fprintf(stderr, "bad arguments\n"); return 2; }
-    std::vector<std::shared_ptr<Competitors::GPUAmd>> comps;
+    std::vector<CompetitorPtr> comps;
+    comps.push_back(std::make_shared<Competitors::CPUHost>());      // competitors[0]: the ground truth
     for (int st : {SDDMM_EXACT, SDDMM_AUTO, SDDMM_FLAT, SDDMM_ROW_WAVE, SDDMM_SHORT_ROWS, SDDMM_LDS_TILED, SDDMM_MFMA_TILE})
         comps.push_back(std::make_shared<Competitors::GPUAmd>(st));
     if (header)

@@ -264,18 +264,3 @@ def make(name, size="full", **overrides):
     kw.update(overrides)
     return gen(**kw)
 
-
-if __name__ == "__main__":
-    # python -m dphpc_amd.workloads NAME [--size small] --dump-col FILE
-    # writes the column array of a shape as raw int32 (an index stream for the
-    # row-gather yardstick csrc/gather_probe.hip) and prints its dimensions
-    import argparse
-
-    ap = argparse.ArgumentParser()
-    ap.add_argument("name", choices=sorted(CONFIGS))
-    ap.add_argument("--size", default="full", choices=["full", "small"])
-    ap.add_argument("--dump-col", required=True)
-    args = ap.parse_args()
-    w = make(args.name, args.size)
-    np.ascontiguousarray(w.col, np.int32).tofile(args.dump_col)
-    print("%s: M=%d N=%d nnz=%d columns -> %s" % (args.name, w.M, w.N, len(w.col), args.dump_col))

@@ -15,6 +15,7 @@
 #include <string>
 #include <vector>
 
+#include "cpu_host.hpp"
 #include "gpu_amd.hpp"
 #include "datasets.hpp"
 
@@ -228,6 +229,50 @@ static void cpu_cases() {
         for (int j = 0; j < 240; ++j) shape = shape && u.S_csr.getColPositions()[j] == j % 24 && u.S_csr.getValues()[j] == 1.f;
         CHECK(shape);
         CHECK(u.S_coo.getRowPositions()[239] == 9 && u.A.getRows() == 40 && u.B.getRows() == 24);
+    }
+    {
+        CASE("the driver's CPU-Basic competitor equals the oracle bit for bit (CSR and COO)");
+        // the ground truth of sddmm_driver (cpu_host.hpp) against the closed form of the
+        // reference's sddmm_coo1 (tests/matrix_test.cc:124-137) and against the oracle on
+        // signed random inputs, through the competitor interface like any other competitor
+        Competitors::CPUHost cpu;
+        CHECK(cpu.name == "CPU-Basic" && cpu.csr_supported() && cpu.coo_supported() && !cpu.is_gpu());
+        {
+            Dense<float> A = dense_of({{1, 2}, {3, 4}}), B = dense_of({{-1, 2}, {-3, 4}});
+            Trips t = {{0, 0, 1.f}, {0, 1, 1.f}, {1, 0, 1.f}, {1, 1, 1.f}};
+            COO<float> S(2, 2, t), P(S);
+            P.clearValues();
+            cpu.init_coo(A, B, S, P); cpu.run_coo(A, B, S, P); cpu.cleanup_coo(A, B, S, P);
+            CHECK((P.getValues() == std::vector<float>{3.f, 5.f, 5.f, 7.f}));
+        }
+        std::mt19937_64 rng(4242);
+        for (int K : {1, 7, 32, 100}) {
+            Trips t = random_triplets(rng, 57, 43, 0.2, -1.f, 1.f);
+            COO<float> S_coo(57, 43, t);
+            CSR<float> S(S_coo);
+            Dense<float> A = random_dense(rng, 57, K, -1.f, 1.f), B = random_dense(rng, 43, K, -1.f, 1.f);
+            std::vector<float> ref(S.getValues().size());
+            oracle_sddmm_csr_f32(S.getRows(), K, S.getRowPositions().data(), S.getColPositions().data(), S.getValues().data(),
+                                 A.get_pointer(), B.get_pointer(), ref.data());
+            CSR<float> P(S);
+            P.clearValues();
+            cpu.init_csr(A, B, S, P); cpu.run_csr(A, B, S, P); cpu.cleanup_csr(A, B, S, P);
+            CHECK(P.getValues().size() == ref.size() &&
+                  std::memcmp(P.getValues().data(), ref.data(), ref.size() * sizeof(float)) == 0);
+            CHECK(P.getColPositions() == S.getColPositions() && P.getRowPositions() == S.getRowPositions());
+            COO<float> Pc(S_coo);
+            Pc.clearValues();
+            cpu.init_coo(A, B, S_coo, Pc); cpu.run_coo(A, B, S_coo, Pc); cpu.cleanup_coo(A, B, S_coo, Pc);
+            CHECK(Pc.getValues().size() == ref.size() &&
+                  std::memcmp(Pc.getValues().data(), ref.data(), ref.size() * sizeof(float)) == 0);
+            std::vector<double> mag(ref.size());
+            oracle_sddmm_csr_f64(S.getRows(), K, S.getRowPositions().data(), S.getColPositions().data(), S.getValues().data(),
+                                 A.get_pointer(), B.get_pointer(), nullptr, mag.data());
+            const std::vector<double> got_mag = Competitors::CPUHost::magnitudes(A, B, S);
+            bool same = got_mag.size() == mag.size();
+            for (size_t i = 0; same && i < mag.size(); ++i) same = std::fabs(got_mag[i] - mag[i]) <= 1e-12 * (1.0 + mag[i]);
+            CHECK(same);
+        }
     }
 }
 

@@ -108,3 +108,42 @@ def test_fused_unsupported_and_state(engine_factory):
     want = np.stack([(A[0] @ A[1]) * A[1], (A[1] @ A[0]) * A[0]]).astype(f32)
     np.testing.assert_allclose(out, want, rtol=1e-6, atol=1e-6)
     e.close()
+
+
+def test_fused_non_finite_rows_of_b_stay_in_their_own_entries(engine_factory):
+    """Global entry 0 and the last entry of a long row point at B rows that hold an
+    infinity and a NaN.  Steps past the end of a row work on clamped positions (entry 0
+    for an empty row, the row's last entry otherwise): nothing of those B rows may reach
+    the output row of another row, or turn into inf * 0 inside its own."""
+    rng = np.random.default_rng(77)
+    M, N, K = 70, 400, 32
+    rows = [np.sort(rng.choice(N - 2, int(n), replace=False)) for n in rng.integers(1, 40, M)]
+    rows[0] = np.array([N - 2])                              # entry 0 of the matrix -> B row N-2
+    rows[5] = np.zeros(0, np.int64)                          # empty rows share wavefronts with the others
+    rows[6] = np.zeros(0, np.int64)
+    rows[9] = np.sort(np.concatenate([rng.choice(N - 2, 129, replace=False), [N - 1]]))   # long row ends in B row N-1
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    B[N - 2, 3] = np.inf
+    B[N - 1, 11] = np.nan
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    got_o = e.run_fused()
+    got_p = e.values()
+    with np.errstate(all="ignore"):
+        ref_p, ref_o = O.fusedmm_csr(rowptr, col, val, A, B)
+    rows_of = np.repeat(np.arange(M), lens)
+    bad_entry = (col == N - 2) | (col == N - 1)
+    assert np.array_equal(~np.isfinite(got_p), bad_entry)
+    bad_row = np.zeros(M, bool)
+    bad_row[rows_of[bad_entry]] = True
+    assert np.array_equal(~np.isfinite(got_o).all(axis=1), bad_row), np.nonzero(~np.isfinite(got_o).all(axis=1))
+    assert not got_o[5].any() and not got_o[6].any()
+    clean = ~bad_row
+    np.testing.assert_allclose(got_o[clean], ref_o[clean], rtol=1e-4, atol=1e-5)
+    e.close()
