@@ -2,13 +2,25 @@
 """SDDMM benchmark on one MI355X: GFLOP/s (2*nnz*K) on the FEM-banded fp32 K=32 shape.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--K K] [--strategy S]
+                    [--per-config full|small|none] [--no-cpu]
 
 A step is one SDDMM over the whole sampling matrix with every operand already
-resident in HBM.  Prints ONE JSON line.  The result is validated against the CPU
-oracle before anything is timed; `cpu_baseline` times the reference CPU loop on
-the host cores of the same box in the same run.
+resident in HBM.  Prints ONE JSON line.  The headline (`value`, `roofline`) is the
+workload named on the command line (default: fem_banded, K=32, AUTO); `per_config`
+repeats the measurement for every benchmark shape at full size with its K sweep:
+AUTO and every fixed strategy, launches in a loop ("warm") and launches that follow a
+1 GiB copy through the caches ("cold"), each result read back AFTER its timed
+launches and validated against the CPU oracle, with the reference's CPU loop timed on
+the host cores of the same box beside it.
+
+Roofline figures divide the COMPULSORY bytes of a launch (every operand byte once:
+4(M+1) + 12 nnz + e K (rows_nonempty + columns_touched)) by the launch duration, so a
+kernel that reuses gathered rows cannot exceed the 8 TB/s peak by counting bytes it
+never moved; the gathered-bytes model (one B row per stored entry) is reported apart
+as `gathered_equiv_gbs`.
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -22,12 +34,19 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# the five benchmark shapes with their K sweeps
+PER_CONFIG = [("small_uniform", 32), ("fem_banded", 32), ("fem_banded", 128), ("power_law", 32),
+              ("mixed_density", 32), ("mixed_density", 64), ("mixed_density", 256),
+              ("dense_tiles", 128), ("dense_tiles", 512)]
+FIXED = ["FLAT", "ROW_WAVE", "SHORT_ROWS", "LDS_TILED", "MFMA_TILE"]
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(w, budget_s=20.0):
+# --------------------------------------------------------------------------- CPU side
+def cpu_baseline(w, budget_s=20.0, reps=3):
     """Reference CPU loop (1 thread, as the reference is serial) on the same inputs.
     The whole workload is one sample when a run fits the budget, else a leading
     block of rows.  Returns the dict for the JSON line plus an all-cores figure."""
@@ -42,23 +61,23 @@ def cpu_baseline(w, budget_s=20.0):
     nn = int(rp[-1])
     cc, sv = np.ascontiguousarray(col[:nn]), np.ascontiguousarray(sval[:nn])
     flops = 2.0 * nn * w.K
-    sample = "rows [0,%d) of %d: %d of %d entries, best of 3" % (rows, w.M, nn, w.nnz)
+    sample = "rows [0,%d) of %d: %d of %d entries, best of %d" % (rows, w.M, nn, w.nnz, reps)
     kind = "port"
     best = None
     if O.Ref.available():
         # the reference's own CPUBasic<float>::run_csr compiled from its headers
         kind = "reference"
         coo_r = np.repeat(np.arange(rows, dtype=np.int32), np.diff(rp)).astype(np.int32)
-        best, _ = O.Ref().cpu_basic_csr_seconds(rows, w.N, coo_r, cc, sv, w.A[:rows], w.B, reps=3)
+        best, _ = O.Ref().cpu_basic_csr_seconds(rows, w.N, coo_r, cc, sv, w.A[:rows], w.B, reps=reps)
     else:
-        for _ in range(3):
+        for _ in range(reps):
             t0 = time.perf_counter()
             O.sddmm_csr(rp, cc, sv, w.A, w.B, threads=1)
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
     threads = O.max_threads()
     allc = None
-    for _ in range(3):
+    for _ in range(reps):
         t0 = time.perf_counter()
         O.sddmm_csr(rp, cc, sv, w.A, w.B, threads=threads)
         dt = time.perf_counter() - t0
@@ -68,9 +87,24 @@ def cpu_baseline(w, budget_s=20.0):
              "sample": sample})
 
 
+class Checker:
+    """The CPU oracle's result for one workload, computed once (all host cores)."""
+
+    def __init__(self, w):
+        from oracle import oracle as O
+        self.O = O
+        self.ref = O.sddmm_csr(w.rowptr, w.col, w.sval, w.A, w.B, threads=0)
+        _, self.mag = O.sddmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+
+    def check(self, got, rtol):
+        ok, worst, i = self.O.check_values_fast(got, self.ref, mag=self.mag, rtol=rtol)
+        return ok, worst, i
+
+
 def load_traffic(key):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
-    recorded by hand in profiles/traffic.json; None when not measured."""
+    """HBM bytes per launch from an earlier rocprofv3 --pmc pair of runs (FETCH_SIZE,
+    WRITE_SIZE), recorded by hand in profiles/traffic.json: a constant of the
+    repository, NOT measured by this run; None when there is no record."""
     p = os.path.join(ROOT, "profiles", "traffic.json")
     if not os.path.exists(p):
         return None
@@ -80,31 +114,154 @@ def load_traffic(key):
         return None
 
 
-def cold_launches(engine, reps):
-    """Median device time of a launch right after 1 GiB has been copied through the
-    caches (two 512 MiB device buffers, copied with the HIP runtime); None when the
-    runtime calls are not available."""
-    import ctypes as C
-    try:
-        hip = C.CDLL("libamdhip64.so")
-        hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
-        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
-        hip.hipFree.argtypes = [C.c_void_p]
-        n = 512 << 20
-        a, b = C.c_void_p(), C.c_void_p()
-        if hip.hipMalloc(C.byref(a), n) != 0 or hip.hipMalloc(C.byref(b), n) != 0:
+# --------------------------------------------------------------------------- GPU side
+class CacheFlusher:
+    """Two 512 MiB device buffers: copying one onto the other (1 GiB through the
+    caches; the last-level cache holds 256 MB) leaves nothing of the SDDMM operands
+    in any cache level."""
+
+    def __init__(self):
+        self.ok = False
+        try:
+            self.hip = C.CDLL("libamdhip64.so")
+        except OSError:
+            return
+        self.hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        self.hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        self.hip.hipFree.argtypes = [C.c_void_p]
+        self.n = 512 << 20
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        if self.hip.hipMalloc(C.byref(self.a), self.n) != 0:
+            return
+        if self.hip.hipMalloc(C.byref(self.b), self.n) != 0:
+            self.hip.hipFree(self.a)
+            return
+        self.ok = True
+
+    def cold_launches(self, engine, reps):
+        """Median device time (ms) of a launch right after the flush; None when unavailable."""
+        if not self.ok:
             return None
         times = []
         for _ in range(reps):
-            if hip.hipMemcpy(b, a, n, 3) != 0:          # device to device, returns when done
+            if self.hip.hipMemcpy(self.b, self.a, self.n, 3) != 0:      # device to device, returns when done
                 break
-            hip.hipDeviceSynchronize()
+            self.hip.hipDeviceSynchronize()
             times.append(float(engine.time_runs(0, 1)[0]))
-        hip.hipFree(a)
-        hip.hipFree(b)
         return float(np.median(times)) if times else None
-    except OSError:
-        return None
+
+    def close(self):
+        if self.ok:
+            self.hip.hipFree(self.a)
+            self.hip.hipFree(self.b)
+            self.ok = False
+
+
+def upload(e, w, capi):
+    if w.dtype != "f32":
+        e.set_dense(w.A_bits, w.B_bits, capi.BF16 if w.dtype == "bf16" else capi.F16)
+    else:
+        e.set_dense(w.A, w.B, capi.F32)
+
+
+def rtol_for(w, strategy_name):
+    # 16-bit operands on the tile path are allowed 1e-2 (fp32 accumulation of exact products
+    # lands far inside it); everything else is held to 1e-5
+    return 1e-2 if w.dtype != "f32" and strategy_name == "MFMA_TILE" else 1e-5
+
+
+def time_strategy(e, w, capi, name, steps, warmup, flusher, checker, cold_reps=6):
+    """Plan `name`, run warm and cold launches, then read P back and validate it.
+    The pattern is set again first, which clears P: what is validated is what the
+    timed launches wrote.  Returns a dict, or {"error": ...} when the strategy does not
+    apply to this input."""
+    strategy = capi.STRATEGY_NAMES.index(name)
+    try:
+        e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+        e.plan(strategy)
+        st = e.stats()
+        plan_ms = st.plan_ms
+        for _ in range(warmup):
+            e.launch()
+        e.synchronize()
+        region = min(e.time_region(steps) for _ in range(3))
+        warm_ms = region / steps
+        cold_ms = flusher.cold_launches(e, cold_reps) if flusher is not None else None
+        st = e.stats()
+        out = {"us": warm_ms * 1e3, "cold_us": None if cold_ms is None else cold_ms * 1e3,
+               "plan_us": plan_ms * 1e3, "resolved": capi.STRATEGY_NAMES[st.strategy_used],
+               "launches": st.kernels_launched or 1}
+        if checker is not None:
+            got = e.values()
+            ok, worst, i = checker.check(got, rtol_for(w, name))
+            if not ok:
+                log("VALIDATION FAILED: %s K=%d %s entry %d got %r ref %r (%.2f x tolerance)" % (
+                    w.name, w.K, name, i, got[i], checker.ref[i], worst))
+                sys.exit(1)
+            out["validated"] = {"entries": int(len(got)), "worst_over_tol": round(worst, 4)}
+        if name == "AUTO":
+            out["classes"] = {"rows_short": st.rows_short, "rows_medium": st.rows_medium, "rows_long": st.rows_long,
+                              "panels": st.panels, "nnz_panel": st.nnz_panel, "mfma_tiles": st.mfma_tiles,
+                              "nnz_mfma": st.nnz_mfma}
+        return out
+    except capi.SddmmError as ex:
+        if ex.code == capi.ERR_UNSUPPORTED:
+            return {"error": "unsupported"}
+        raise
+
+
+def fractions(w, us, cold_us):
+    """Compulsory bytes over launch time against the HBM peak (and the dense-tile
+    shape's flops against the bf16 MFMA peak)."""
+    comp = w.bytes_compulsory()
+    d = {"frac": comp / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+         "frac_cold": None if not cold_us else comp / (cold_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    if w.dtype != "f32":
+        d["mfma_frac"] = w.flops() / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS
+    return d
+
+
+def per_config_entry(name, K, capi, workloads, steps, warmup, flusher, no_cpu, size="full"):
+    t0 = time.time()
+    w = workloads.make(name, size, K=K)
+    checker = Checker(w)
+    e = capi.Engine(0)
+    upload(e, w, capi)
+    auto = time_strategy(e, w, capi, "AUTO", steps, warmup, flusher, checker)
+    fixed = {s: time_strategy(e, w, capi, s, steps, warmup, flusher, checker) for s in FIXED}
+    e.close()
+    ran = {s: r for s, r in fixed.items() if "us" in r}
+    best = min(ran, key=lambda s: ran[s]["us"])
+    best_cold = min(ran, key=lambda s: ran[s]["cold_us"] or float("inf"))
+    entry = {
+        "workload": w.name, "K": w.K, "dtype": w.dtype, "M": w.M, "N": w.N, "nnz": w.nnz,
+        "auto_us": auto["us"], "auto_cold_us": auto["cold_us"], "auto_resolved": auto["resolved"],
+        "plan_us": auto["plan_us"], "launches": auto["launches"],
+        "best_fixed": best, "best_fixed_us": ran[best]["us"],
+        "best_fixed_cold": best_cold, "best_fixed_cold_us": ran[best_cold]["cold_us"],
+        "auto_over_best_fixed": ran[best]["us"] / auto["us"],
+        "fixed_us": {s: (round(r["us"], 2) if "us" in r else r["error"]) for s, r in fixed.items()},
+        "gflops": w.flops() / (auto["us"] * 1e-6) / 1e9,
+        "bytes_compulsory": w.bytes_compulsory(),
+        "compulsory_gbs": w.bytes_compulsory() / (auto["us"] * 1e-6) / 1e9,
+        "gathered_equiv_gbs": w.bytes_gathered() / (auto["us"] * 1e-6) / 1e9,
+        "classes": auto.get("classes"),
+        "validated": {"strategies": 1 + len(ran), "entries": w.nnz,
+                      "worst_over_tol": max([auto["validated"]["worst_over_tol"]] +
+                                            [r["validated"]["worst_over_tol"] for r in ran.values()])},
+    }
+    entry.update(fractions(w, auto["us"], auto["cold_us"]))
+    if not no_cpu:
+        base, allc = cpu_baseline(w, budget_s=1.5, reps=2)
+        entry["cpu_1core_gflops"] = round(base["value"], 3)
+        entry["cpu_1core_kind"] = base["kind"]
+        entry["cpu_allcores_gflops"] = round(allc["value"], 2)
+        entry["cpu_cores"] = allc["cores"]
+        entry["cpu_sample"] = base["sample"]
+    log("per_config %s K=%d: AUTO %.1f us (cold %s), best fixed %s %.1f us, frac %.3f  [%.1fs]" % (
+        w.name, w.K, auto["us"], "%.1f" % auto["cold_us"] if auto["cold_us"] else "-", best, ran[best]["us"],
+        entry["frac"], time.time() - t0))
+    return entry
 
 
 def main():
@@ -118,8 +275,11 @@ def main():
     ap.add_argument("--strategy", default="AUTO")
     ap.add_argument("--include-plan", action="store_true", help="re-run the classifier inside every timed step")
     ap.add_argument("--f16", action="store_true", help="dense_tiles: IEEE half operands instead of bf16")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--no-check", action="store_true", help="skip validation against the oracle")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline legs")
+    ap.add_argument("--no-check", action="store_true", help="skip validation of the headline against the oracle")
+    ap.add_argument("--per-config", default=None, choices=["full", "small", "none"],
+                    help="size of the per_config sweep (default: full with --size full, none otherwise)")
+    ap.add_argument("--no-per-config", action="store_true", help="headline only (e.g. under a profiler)")
     args = ap.parse_args()
 
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -135,31 +295,12 @@ def main():
     w = workloads.make(args.workload, args.size, K=args.K, **extra)
     log("workload %s: M=%d N=%d K=%d nnz=%d (%.1fs to generate)" % (w.name, w.M, w.N, w.K, w.nnz, time.time() - t0))
     strategy = capi.STRATEGY_NAMES.index(args.strategy.upper())
-    bf16 = w.dtype != "f32"          # 16-bit operands (bf16 or IEEE half)
 
     e = capi.Engine(0)
-    if bf16:
-        e.set_dense(w.A_bits, w.B_bits, capi.BF16 if w.dtype == "bf16" else capi.F16)
-    else:
-        e.set_dense(w.A, w.B, capi.F32)
-    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    upload(e, w, capi)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)      # P starts at zero
     e.plan(strategy)
     plan_ms = e.stats().plan_ms
-
-    # ---- validate before timing ------------------------------------------------
-    validated = None
-    if not args.no_check:
-        from oracle import oracle as O
-        e.run()
-        got = e.values()
-        ref = O.sddmm_csr(w.rowptr, w.col, w.sval, w.A, w.B, threads=0)
-        _, mag = O.sddmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
-        ok, worst, i = O.check_values(got, ref, mag=mag, rtol=1e-2 if bf16 and strategy == capi.MFMA_TILE else 1e-5)
-        if not ok:
-            log("VALIDATION FAILED: entry %d got %r ref %r (%.2f x tolerance)" % (i, got[i], ref[i], worst))
-            sys.exit(1)
-        validated = {"entries": int(len(got)), "worst_over_tol": round(worst, 4)}
-        log("validated %d entries against the CPU oracle (worst %.3f of tolerance)" % (len(got), worst))
 
     # ---- timed region: W warm-up steps, then exactly K steps --------------------
     for _ in range(args.warmup):
@@ -176,27 +317,52 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
 
+    # ---- validate what the timed launches left in P ------------------------------
+    validated = None
+    if not args.no_check:
+        got = e.values()
+        ok, worst, i = Checker(w).check(got, rtol_for(w, args.strategy.upper()))
+        if not ok:
+            log("VALIDATION FAILED: entry %d got %r (%.2f x tolerance)" % (i, got[i], worst))
+            sys.exit(1)
+        validated = {"entries": int(len(got)), "worst_over_tol": round(worst, 4), "when": "after the timed steps"}
+        log("validated %d entries against the CPU oracle (worst %.3f of tolerance)" % (len(got), worst))
+
     # ---- device time from HIP events on the launch stream ------------------------
     # average launch duration: the same K steps between one pair of events (best of 3
     # regions; what a kernel trace of this loop reports per launch); `isolated` is
     # each launch between its own events with a wait in between, i.e. with the idle
-    # gap and cold start a lone launch pays
+    # gap a lone launch pays; `cold` is a launch that follows a 1 GiB device copy
     region = min(e.time_region(args.steps, include_plan=args.include_plan) for _ in range(3))
     ev_avg = region / args.steps
     ev = e.time_runs(2, max(args.steps, 20), include_plan=args.include_plan)
     ev_p50, ev_min = float(np.median(ev)), float(ev.min())
-    # a launch that finds nothing of its operands in the caches: 1 GiB is copied on the
-    # device before each of these launches (the last-level cache holds 256 MB)
-    ev_cold = None
-    if not args.include_plan:
-        ev_cold = cold_launches(e, 10)
+    flusher = CacheFlusher()
+    ev_cold = None if args.include_plan else flusher.cold_launches(e, 10)
     # classifier + run in one timed region, for the record (the classifier belongs to
     # the init phase, as the reference's preprocessing does: benchmark.hpp:148-190
     # times init_csr apart from run_csr)
     ev_plan = e.time_runs(1, 5, include_plan=True)
     st = e.stats()
-    flops, gathered = w.flops(), w.bytes_gathered()
-    achieved = gathered / (ev_avg * 1e-3) / 1e9
+    flops, gathered, compulsory = w.flops(), w.bytes_gathered(), w.bytes_compulsory()
+    achieved = compulsory / (ev_avg * 1e-3) / 1e9
+    achieved_cold = None if not ev_cold else compulsory / (ev_cold * 1e-3) / 1e9
+    traffic = load_traffic("%s_K%d_%s" % (w.name, w.K, w.dtype))
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBS,
+                "bytes": "compulsory: every operand byte once per launch",
+                "achieved_cold": achieved_cold,
+                "frac_cold": None if achieved_cold is None else achieved_cold / HBM_PEAK_GBS,
+                "gathered_equiv_gbs": gathered / (ev_avg * 1e-3) / 1e9,
+                "traffic": traffic,
+                "traffic_source": None if traffic is None else
+                "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this "
+                "command, a recorded constant, not measured by this run"}
+    if traffic:
+        roofline["traffic_frac"] = traffic / (ev_avg * 1e-3) / 1e9 / HBM_PEAK_GBS
+        roofline["traffic_frac_cold"] = None if not ev_cold else traffic / (ev_cold * 1e-3) / 1e9 / HBM_PEAK_GBS
+    if w.dtype != "f32":
+        roofline["mfma_frac"] = flops / (ev_avg * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
 
     out = {
         "metric": "SDDMM GFLOP/s (2*nnz*K), 1 MI355X, K=%d" % w.K,
@@ -214,14 +380,13 @@ def main():
         "config": {"workload": w.name, "size": args.size, "M": w.M, "N": w.N, "K": w.K, "nnz": w.nnz,
                    "strategy": capi.STRATEGY_NAMES[st.strategy_used], "requested": args.strategy.upper(),
                    "plan_in_step": bool(args.include_plan)},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": load_traffic("%s_K%d_%s" % (w.name, w.K, w.dtype))},
+        "roofline": roofline,
         "kernel_ms": {"avg": ev_avg, "isolated_p50": ev_p50, "isolated_min": ev_min, "cold_p50": ev_cold,
                       "launches_per_step": st.kernels_launched or 1},
         "gflops_kernel": flops / (ev_avg * 1e-3) / 1e9,
+        "gflops_kernel_cold": None if not ev_cold else flops / (ev_cold * 1e-3) / 1e9,
         "bytes_gathered": gathered,
-        "bytes_compulsory": w.bytes_compulsory(),
+        "bytes_compulsory": compulsory,
         "plan_ms": plan_ms,
         "plan_plus_run_ms": float(np.median(ev_plan)),
         "classes": {"rows_short": st.rows_short, "rows_medium": st.rows_medium, "rows_long": st.rows_long,
@@ -229,11 +394,19 @@ def main():
                     "nnz_mfma": st.nnz_mfma},
         "validated": validated,
     }
+    e.close()
     if not args.no_cpu:
         base, allc = cpu_baseline(w)
         out["cpu_baseline"] = base
         out["cpu_allcores"] = allc
-    e.close()
+    sweep = args.per_config or ("full" if args.size == "full" else "none")
+    if not args.no_per_config and sweep != "none":
+        t0 = time.time()
+        out["per_config_size"] = sweep
+        out["per_config"] = [per_config_entry(n, k, capi, workloads, max(20, min(args.steps, 50)), 3, flusher,
+                                              args.no_cpu, sweep) for n, k in PER_CONFIG]
+        log("per_config: %d entries in %.0f s" % (len(out["per_config"]), time.time() - t0))
+    flusher.close()
     print(json.dumps(out), flush=True)
 
 

@@ -65,6 +65,8 @@ def lib():
         L.oracle_density.argtypes = [C.c_int, C.c_int, C.c_int64]
         L.oracle_density.restype = C.c_double
         L.oracle_max_threads.restype = C.c_int
+        L.oracle_compare.argtypes = [C.c_int64, _f32p, _f32p, C.c_void_p, C.c_double, C.c_double, C.POINTER(C.c_int64)]
+        L.oracle_compare.restype = C.c_double
         _lib = L
     return _lib
 
@@ -213,6 +215,21 @@ def check_values(got, ref, mag=None, rtol=1e-5, floor=0.25):
     ratio = np.nan_to_num(ratio, nan=np.inf, posinf=np.inf)
     i = int(np.argmax(ratio))
     return bool(ratio[i] <= 1.0), float(ratio[i]), i
+
+
+def check_values_fast(got, ref, mag=None, rtol=1e-5, floor=0.25):
+    """`check_values` for large fp32 arrays: the same test in C on all cores
+    (oracle_compare); tests/test_oracle.py holds the two to the same answers."""
+    got, ref = _c(got, np.float32), _c(ref, np.float32)
+    if got.shape != ref.shape:
+        return False, np.inf, -1
+    if got.size == 0:
+        return True, 0.0, -1
+    m = None if mag is None else _c(mag, np.float64)
+    at = C.c_int64(-1)
+    worst = lib().oracle_compare(got.size, got.ravel(), ref.ravel(), None if m is None else m.ctypes.data_as(C.c_void_p),
+                                 float(rtol), float(floor), C.byref(at))
+    return bool(worst <= 1.0), float(worst), int(at.value)
 
 
 class Ref:

@@ -18,6 +18,9 @@
  *   oracle_dispatch           matrices/CSR.hpp:196-264
  *   oracle_density            matrices/CSR.hpp:157-159 (in 64-bit; the reference
  *                             multiplies rows*cols in int and overflows above 46340^2)
+ *   oracle_compare            no counterpart (a comparator, not arithmetic): the value
+ *                             test of oracle.check_values over large arrays, held to
+ *                             the numpy version by tests/test_oracle.py
  *   oracle_fusedmm_csr_f32/_f64   no counterpart: the reference stops at P.  SpMM of
  *                             the SDDMM result with B, written in the reference's
  *                             style (multiply, then add, entries in storage order);
@@ -299,4 +302,36 @@ int oracle_dispatch(int rows, const int32_t *rowptr, int parts, int stride, int3
     while (w <= parts) start_idx[w++] = rows;       /* idle parts */
     free(sizes);
     return w;
+}
+
+/* ---- comparator --------------------------------------------------------- */
+/* ratio[i] = 0 when got[i] == ref[i], else |got-ref| / (rtol * max(|ref|, floor*mag[i]))
+ * (mag may be NULL); a NaN ratio counts as infinite.  Returns the largest ratio and
+ * the first position that attains it: the test passes when it is <= 1. */
+double oracle_compare(int64_t n, const float *got, const float *ref, const double *mag,
+                      double rtol, double floor_, int64_t *worst_at)
+{
+    double worst = -1.0;
+    int64_t at = -1;
+#pragma omp parallel
+    {
+        double w = -1.0;
+        int64_t a = -1;
+#pragma omp for schedule(static) nowait
+        for (int64_t i = 0; i < n; i++) {
+            const double g = (double)got[i], r = (double)ref[i];
+            double scale = fabs(r);
+            if (mag && floor_ * mag[i] > scale) scale = floor_ * mag[i];
+            const double err = fabs(g - r);
+            double ratio = err == 0.0 ? 0.0 : err / (rtol * scale);
+            if (isnan(ratio)) ratio = INFINITY;
+            if (ratio > w) { w = ratio; a = i; }
+        }
+#pragma omp critical
+        {
+            if (w > worst || (w == worst && a >= 0 && (at < 0 || a < at))) { worst = w; at = a; }
+        }
+    }
+    if (worst_at) *worst_at = at;
+    return n > 0 ? worst : 0.0;
 }

@@ -27,7 +27,8 @@ def test_traffic_table_names_existing_profiles():
 
 @pytest.mark.gpu
 def test_json_line_on_a_small_run():
-    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--size", "small", "--steps", "5", "--warmup", "2"],
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--size", "small", "--steps", "5", "--warmup", "2",
+                        "--per-config", "small"],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=280)
     assert p.returncode == 0, p.stderr
     lines = [l for l in p.stdout.splitlines() if l.strip()]
@@ -42,6 +43,19 @@ def test_json_line_on_a_small_run():
     r = d["roofline"]
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-12
+    # compulsory bytes over launch time: a fraction of the peak, whatever the kernel reuses
+    assert 0 < r["frac"] <= 1.0 and r["gathered_equiv_gbs"] >= r["achieved"]
+    assert r["achieved"] == pytest.approx(d["bytes_compulsory"] / (d["kernel_ms"]["avg"] * 1e-3) / 1e9)
     c = d["cpu_baseline"]
     assert c["kind"] in ("reference", "port") and c["cores"] == 1 and c["value"] > 0 and c["sample"]
     assert d["validated"]["entries"] == d["config"]["nnz"]
+    # the sweep over the five shapes: AUTO next to every fixed strategy, all validated
+    pc = d["per_config"]
+    assert [(x["workload"], x["K"]) for x in pc] == [
+        ("small_uniform", 32), ("fem_banded", 32), ("fem_banded", 128), ("power_law", 32), ("mixed_density", 32),
+        ("mixed_density", 64), ("mixed_density", 256), ("dense_tiles", 128), ("dense_tiles", 512)]
+    for x in pc:
+        assert 0 < x["frac"] <= 1.0 and x["auto_us"] > 0 and x["best_fixed"] in x["fixed_us"]
+        assert x["validated"]["entries"] == x["nnz"] and x["validated"]["worst_over_tol"] <= 1.0
+        assert x["cpu_1core_gflops"] > 0
+        assert x["dtype"] == ("bf16" if x["workload"] == "dense_tiles" else "f32")

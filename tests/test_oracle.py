@@ -305,6 +305,37 @@ def test_comparator():
     assert not ok                                     # sign error is caught (the reference's == would pass it)
 
 
+def test_fast_comparator_gives_the_answers_of_the_numpy_one():
+    """oracle_compare (C, all cores; what bench.py uses on tens of millions of entries)
+    against check_values on exact matches, small and large errors, zero references with
+    and without a magnitude floor, NaN and infinities on either side."""
+    rng = np.random.default_rng(5)
+    n = 200_003
+    ref = rng.uniform(-1, 1, n).astype(f32)
+    ref[::97] = 0
+    mag = np.abs(ref).astype(np.float64) + rng.random(n)
+    cases = []
+    cases.append(ref.copy())
+    g = ref.copy(); g[1234] *= f32(1 + 2e-5); cases.append(g)
+    g = ref.copy(); g[97 * 5] = f32(1e-7); cases.append(g)
+    g = (ref * (1 + rng.uniform(-4e-6, 4e-6, n))).astype(f32); cases.append(g)
+    g = ref.copy(); g[77] = np.nan; cases.append(g)
+    g = ref.copy(); g[n - 1] = np.inf; g[5] = -np.inf; cases.append(g)
+    for i, got in enumerate(cases):
+        for m in (None, mag):
+            for rtol in (1e-5, 1e-2):
+                a = O.check_values(got, ref, mag=m, rtol=rtol)
+                b = O.check_values_fast(got, ref, mag=m, rtol=rtol)
+                assert a[0] == b[0] and a[2] == b[2], (i, m is None, rtol, a, b)
+                assert a[1] == b[1] or abs(a[1] - b[1]) <= 1e-12 * abs(a[1]), (i, a, b)
+    bad_ref = ref.copy(); bad_ref[10] = np.inf
+    got = bad_ref.copy()
+    a, b = O.check_values(got, bad_ref, mag=mag), O.check_values_fast(got, bad_ref, mag=mag)
+    assert a[0] == b[0] and a[2] == b[2] and not a[0]          # inf - inf is NaN: never passes
+    assert O.check_values_fast(np.zeros(0, f32), np.zeros(0, f32)) == (True, 0.0, -1)
+    assert O.check_values_fast(np.zeros(3, f32), np.zeros(4, f32))[0] is False
+
+
 # ---- SDDMM followed by SpMM (no counterpart in the reference: pinned by identities) ----
 def test_fusedmm_oracle_against_dense_algebra():
     """O = (S o (A B^T)) B.  Brute force in float64 on small inputs, the all-ones S
