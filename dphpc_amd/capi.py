@@ -18,6 +18,8 @@ F32, BF16, F16 = 0, 1, 2
 
 OK, ERR_INVALID, ERR_NULL, ERR_STATE, ERR_ALLOC, ERR_HIP, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_PATTERN = (
     0, -1, -2, -3, -4, -5, -6, -7, -8)
+ERR_TOO_LARGE = -9
+NOALLOC_MAX_NNZ = 1 << 24
 
 # every symbol include/sddmm_amd.h declares
 EXPORTS = [
@@ -27,6 +29,7 @@ EXPORTS = [
     "sddmm_launch", "sddmm_synchronize", "sddmm_time_runs", "sddmm_time_region", "sddmm_run_fused",
     "sddmm_get_fused", "sddmm_get_fused_device", "sddmm_get_values",
     "sddmm_get_values_device", "sddmm_last_stats", "sddmm_partition_rows", "sddmm_version",
+    "sddmm_launch_noalloc",
 ]
 
 
@@ -99,6 +102,7 @@ def load_library():
     L.sddmm_last_stats.argtypes = [vp, C.POINTER(Stats)]
     L.sddmm_partition_rows.argtypes = [i32, vp, i32, i32, vp]
     L.sddmm_version.restype = C.c_char_p
+    L.sddmm_launch_noalloc.argtypes = [i32, i32, i32, i64, vp, vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 

@@ -14,6 +14,7 @@
 #include <climits>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -1029,6 +1030,9 @@ const char *sddmm_strerror(int code) {
         case SDDMM_ERR_UNSUPPORTED: return "strategy not applicable";
         case SDDMM_ERR_NO_DEVICE: return "no usable HIP device";
         case SDDMM_ERR_PATTERN: return "malformed sparse structure";
+        case SDDMM_ERR_TOO_LARGE:
+            return "more stored entries than the static scratch buffer of sddmm_launch_noalloc holds "
+                   "(SDDMM_NOALLOC_MAX_NNZ)";
         default: return "unknown error";
     }
 }
@@ -1521,6 +1525,74 @@ int sddmm_get_values_device(sddmm_ctx *c, const float **dP) {
 int sddmm_last_stats(const sddmm_ctx *c, sddmm_stats *out) {
     if (!c || !out) return SDDMM_ERR_NULL;
     *out = c->stats;
+    return SDDMM_OK;
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------
+// The row index per stored entry that the flat kernel reads (k_expand_rows writes it,
+// k_flat reads it) lives in a static device array instead of a hipMalloc'ed buffer.
+// Every device the library runs on holds its own copy of the array at its own address
+// until the process ends; in host code the array's name is only a handle for
+// hipGetSymbolAddress, never an address to hand to a kernel.
+}  // extern "C"
+
+static __device__ __align__(256) int32_t scratch[SDDMM_NOALLOC_MAX_NNZ];
+
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+int32_t *g_scratch_ptr[NOALLOC_MAX_DEVICES] = {nullptr};   // device address of `scratch`, per device
+std::mutex g_scratch_mu;
+
+// Device address of the current device's copy of `scratch` (looked up once per device).
+int scratch_of_current_device(int *device, int32_t **ptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) return SDDMM_ERR_NO_DEVICE;
+    if (dev >= NOALLOC_MAX_DEVICES) return SDDMM_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return SDDMM_ERR_HIP;
+        g_scratch_ptr[dev] = static_cast<int32_t *>(p);
+    }
+    *device = dev;
+    *ptr = g_scratch_ptr[dev];
+    return SDDMM_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, const float *dB,
+                         const int32_t *d_rowptr, const int32_t *d_col, const float *d_sval, float *dP,
+                         void *stream) {
+    if (M < 0 || N < 0 || K < 1 || nnz < 0) return SDDMM_ERR_INVALID;
+    if (nnz > 0 && (M == 0 || N == 0)) return SDDMM_ERR_INVALID;
+    if (nnz > (int64_t)SDDMM_NOALLOC_MAX_NNZ) return SDDMM_ERR_TOO_LARGE;
+    if (!d_rowptr || (nnz > 0 && (!dA || !dB || !d_col || !d_sval || !dP))) return SDDMM_ERR_NULL;
+    if (((uintptr_t)dA | (uintptr_t)dB) & 15) return SDDMM_ERR_INVALID;
+    int device = -1;
+    int32_t *rowidx = nullptr;
+    const int rc = scratch_of_current_device(&device, &rowidx);
+    if (rc) return rc;
+    if (nnz == 0) return SDDMM_OK;
+    // a context on the stack: nothing is allocated for it, it only carries the launch arguments
+    sddmm_ctx c;
+    c.device = device;
+    c.stream = static_cast<hipStream_t>(stream);
+    c.M = M; c.N = N; c.K = K; c.dtype = SDDMM_F32;
+    c.dA = const_cast<float *>(dA);
+    c.dB = const_cast<float *>(dB);
+    c.sM = M; c.sN = N; c.nnz = nnz;
+    c.d_rowptr = const_cast<int32_t *>(d_rowptr);
+    c.d_col = const_cast<int32_t *>(d_col);
+    c.d_sval = const_cast<float *>(d_sval);
+    c.dP = dP;
+    c.d_rowidx = rowidx;                       // every position below nnz is rewritten: nothing to clear
+    SDDMM_LAUNCH(&c, k_expand_rows, grid_for(M, 256), 256, c.d_rowptr, M, rowidx);
+    launch_flat(&c);
+    if (hipGetLastError() != hipSuccess) return SDDMM_ERR_HIP;
+    if (c.oversize) return SDDMM_ERR_UNSUPPORTED;
     return SDDMM_OK;
 }
 

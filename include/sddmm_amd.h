@@ -44,7 +44,8 @@ enum sddmm_status {
     SDDMM_ERR_HIP = -5,         /* a HIP runtime call or kernel launch failed        */
     SDDMM_ERR_UNSUPPORTED = -6, /* strategy not applicable to these operands         */
     SDDMM_ERR_NO_DEVICE = -7,   /* no usable gfx950 device                           */
-    SDDMM_ERR_PATTERN = -8      /* CSR/COO structure is malformed (see sddmm_set_*)  */
+    SDDMM_ERR_PATTERN = -8,     /* CSR/COO structure is malformed (see sddmm_set_*)  */
+    SDDMM_ERR_TOO_LARGE = -9    /* sddmm_launch_noalloc: nnz > SDDMM_NOALLOC_MAX_NNZ */
 };
 
 enum sddmm_dtype {
@@ -182,6 +183,30 @@ int sddmm_time_runs(sddmm_ctx *ctx, int warmup, int reps, int include_plan, floa
  * (what a kernel trace of the same loop reports), without the idle gap that the
  * per-launch synchronisation of sddmm_time_runs puts in front of every launch. */
 int sddmm_time_region(sddmm_ctx *ctx, int reps, int include_plan, float *total_ms);
+
+/* ---- one launch that allocates nothing ----------------------------------------- */
+/* No counterpart in the reference.  For callers that cannot call hipMalloc: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid allocation.  One complete
+ * fp32 SDDMM on caller-owned device buffers, enqueued on `stream` (a hipStream_t of the
+ * current device, NULL = the null stream) without waiting, like sddmm_launch on a context
+ * planned with SDDMM_FLAT over sddmm_set_dense_device / sddmm_set_csr_device operands --
+ * same kernels, bit-identical values -- except that the row index per stored entry which
+ * the flat kernel reads is written into a static device array of the library
+ * (SDDMM_NOALLOC_MAX_NNZ int32 = 64 MiB per device, held until the process ends) instead
+ * of an allocated buffer.  It calls no hipMalloc, hipFree or other allocating routine and
+ * waits for nothing.  The first call on a device looks up that device's copy of the
+ * array (hipGetSymbolAddress): make it outside a graph capture (nnz = 0 will do).
+ *   - dA [M x K], dB [N x K] row-major fp32, 16-byte aligned; d_rowptr[M+1], d_col[nnz],
+ *     d_sval[nnz], dP[nnz]; P is complete when `stream` has executed the call;
+ *   - the structure is NOT validated here (that needs a read-back): pass arrays that
+ *     sddmm_set_csr_device would accept;
+ *   - nnz > SDDMM_NOALLOC_MAX_NNZ returns SDDMM_ERR_TOO_LARGE and launches nothing;
+ *   - all calls on one device share the array: calls that may overlap on one GPU
+ *     (different streams, different threads) race; order them on one stream. */
+#define SDDMM_NOALLOC_MAX_NNZ (1 << 24)
+int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, const float *dB,
+                         const int32_t *d_rowptr, const int32_t *d_col, const float *d_sval, float *dP,
+                         void *stream);
 
 /* ---- SDDMM followed by SpMM over the same pattern ("FusedMM") -------------- */
 /* O[i,:] = sum over the stored (i,j) of P[i,j] * B[j,:], with P as sddmm_run computes
