@@ -66,17 +66,20 @@ enum sddmm_strategy {
                              (the role of src/competitors/gpu/gpu_convert.cu:8-50)    */
     SDDMM_ROW_WAVE = 2,   /* one wavefront per row segment, A row held in registers   */
     SDDMM_SHORT_ROWS = 3, /* many short rows per wavefront                            */
-    SDDMM_LDS_TILED = 4,  /* row panels: 8 rows with a common column list share every
-                             gathered B row, A rows held in registers; other rows on
-                             AUTO's gather kernels (the role of the row-panel kernels
-                             src/competitors/gpu/gpu_shared.cu:18-88 and
-                             gpu_preprocessing.cu:18-96: B reused across a row panel) */
+    SDDMM_LDS_TILED = 4,  /* ROW PANELS (also spelled SDDMM_ROW_PANEL): 8 rows with a common
+                             column list share every gathered B row, which is held in
+                             registers -- nothing is staged in LDS, the name is the slot of
+                             the reference's LDS-tiled row-panel kernels that this strategy
+                             fills (src/competitors/gpu/gpu_shared.cu:18-88,
+                             gpu_preprocessing.cu:18-96: B reused across a row panel);
+                             other rows run on AUTO's gather kernels                       */
     SDDMM_MFMA_TILE = 5,  /* near-dense 16x16 tiles on MFMA, remainder on AUTO's
                              gather kernels (the role of gpu_tensor.cu:27-99).  AUTO
                              also cuts tiles from the union of the columns of 16
                              similar rows (the active-column lists of
                              gpu_preprocessing.hpp:57-141) and from near-dense rows
                              gathered by column window                                */
+    SDDMM_ROW_PANEL = SDDMM_LDS_TILED,
     SDDMM_EXACT = 6       /* one lane per entry, k ascending, separate fp32 multiply
                              and add: bit-identical to cpu_basic.hpp:18-51            */
 };
