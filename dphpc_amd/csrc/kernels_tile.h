@@ -968,7 +968,77 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
 // of chunk c+2 are being read; every load is issued whatever the position (clamped),
 // so the wait counts stay exact and a group only waits for loads issued four groups
 // earlier.
+//
+// fp32 rows of 128 bytes and more use v_mfma_f32_4x4x1_16b_f32 instead of the 16x16x4
+// shape, whose accumulator the 8 panel rows fill only by half (fp32 MFMA runs at the rate
+// of two plain FMAs per lane, so a half-used 16x16 accumulator is no faster than vector
+// FMAs).  The instruction computes 16 independent 4x4 outer products, block b = lanes
+// 4b..4b+3:  D_b[i][j] += srcA[lane 4b+i] * srcB[lane 4b+j]  (result register i of lane
+// 4b+j).  Blocks are numbered (q, cg): q = k quarter (the 16-byte unit 4s+q of a row, as
+// above), cg = four of the 16 gathered columns.  srcB is the gathered B row of column
+// 4cg+j -- the operand layout of the 16x16 shape, unchanged.  srcA is the panel: with
+// cbsz = 2 the four blocks of one q take srcA from the block that abid names, so the four
+// blocks of a q hold four different things -- block cg: panel rows 4(cg&1).. of unit
+// 4(2s'+(cg>>1))+q -- and one register covers two steps and both row halves: the panel
+// costs STEPS/2 registers of 16 bytes (the 16x16 layout needs STEPS and repeats every
+// row).  Every MFMA does 256 useful multiply-adds.  Results: register i of lane (q,cg,j)
+// is (row i or 4+i, column 4cg+j), partial over q; v_permlane32_swap and
+// v_permlane16_swap add the four k quarters while they deal the row halves and the two
+// groups of a pair out to the lanes, a 4x4 transpose inside every quad (two DPP stages)
+// turns (register = row, lane = column) into (lane = row, register = column): four
+// consecutive entries of a row per lane, which then move to the memory layout as above.
 struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
+
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+template <int ABID>
+__device__ __forceinline__ f32x4_t mfma_blocks(float a, float b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 2, ABID, 0);
+}
+// both row halves of the panel against one component of a gathered unit; AB = 2 * (step parity)
+template <int AB>
+__device__ __forceinline__ void mfma_blocks_unit(const uint4 &r, const uint4 &b, f32x4_t &lo, f32x4_t &hi) {
+    lo = mfma_blocks<AB>(__builtin_bit_cast(float, r.x), __builtin_bit_cast(float, b.x), lo);
+    hi = mfma_blocks<AB + 1>(__builtin_bit_cast(float, r.x), __builtin_bit_cast(float, b.x), hi);
+    lo = mfma_blocks<AB>(__builtin_bit_cast(float, r.y), __builtin_bit_cast(float, b.y), lo);
+    hi = mfma_blocks<AB + 1>(__builtin_bit_cast(float, r.y), __builtin_bit_cast(float, b.y), hi);
+    lo = mfma_blocks<AB>(__builtin_bit_cast(float, r.z), __builtin_bit_cast(float, b.z), lo);
+    hi = mfma_blocks<AB + 1>(__builtin_bit_cast(float, r.z), __builtin_bit_cast(float, b.z), hi);
+    lo = mfma_blocks<AB>(__builtin_bit_cast(float, r.w), __builtin_bit_cast(float, b.w), lo);
+    hi = mfma_blocks<AB + 1>(__builtin_bit_cast(float, r.w), __builtin_bit_cast(float, b.w), hi);
+}
+// a + b where lane l of the result pairs (first, second) as the swap instruction deals them:
+// permlane32_swap: lanes 0..31 get first[l] + first[l+32], lanes 32..63 second[l-32] + second[l]
+__device__ __forceinline__ float swap32_add(float first, float second) {
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned int, first),
+                                                       __builtin_bit_cast(unsigned int, second), false, false);
+    // (element values first: a bit cast applied to a vector element expression reads element 0)
+    const unsigned int x = r.x, y = r.y;
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+}
+// permlane16_swap: even 16-lane rows get first[row] + first[row+1], odd rows second[row-1] + second[row]
+__device__ __forceinline__ float swap16_add(float first, float second) {
+    const u32x2_t r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned int, first),
+                                                       __builtin_bit_cast(unsigned int, second), false, false);
+    const unsigned int x = r.x, y = r.y;
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+}
+// 4x4 transpose inside every quad of lanes: f[i] of lane j  <->  f[j] of lane i
+__device__ __forceinline__ void quad_transpose(float (&f)[4], int lane) {
+    const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
+    {
+        const float t01 = dpp_f32<DPP_QUAD_XOR1>(b0 ? f[0] : f[1]);
+        const float t23 = dpp_f32<DPP_QUAD_XOR1>(b0 ? f[2] : f[3]);
+        f[0] = b0 ? t01 : f[0]; f[1] = b0 ? f[1] : t01;
+        f[2] = b0 ? t23 : f[2]; f[3] = b0 ? f[3] : t23;
+    }
+    {
+        const float t02 = dpp_f32<DPP_QUAD_XOR2>(b1 ? f[0] : f[2]);
+        const float t13 = dpp_f32<DPP_QUAD_XOR2>(b1 ? f[1] : f[3]);
+        f[0] = b1 ? t02 : f[0]; f[2] = b1 ? f[2] : t02;
+        f[1] = b1 ? t13 : f[1]; f[3] = b1 ? f[3] : t13;
+    }
+}
 
 // Wavefronts per workgroup: the launch is a few workgroups per CU (one work item per
 // 8-row panel), so small workgroups spread more evenly over the CUs; measured 2 % faster
@@ -998,15 +1068,26 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
     // S/P layout of a pair of groups: row l>>3, 16-byte unit l&7 of the 128 bytes; units 4..7 are the
     // second group's, whose results sit in lanes 8..15 of every 16
     const int prow = lane >> 3, punit = lane & 7;
-    const int to_memory_from = (16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
+    // fp32 rows of 128 bytes and more: 4x4 blocks, every multiply-add useful (see above)
+    constexpr bool BLOCKS = DT == DT_F32 && STEPS % 2 == 0;
+    const int to_memory_from =
+        (BLOCKS ? 32 * (prow >> 2) + 16 * (punit >> 2) + 4 * (punit & 3) + (prow & 3)
+                : 16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
     constexpr int ROW_UNITS = STEPS * 4;
     // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
     constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
-    // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored
-    uint4 a[STEPS];
-    {
+    constexpr int A_REGS = BLOCKS ? STEPS / 2 : STEPS;
+    uint4 a[A_REGS];
+    if constexpr (BLOCKS) {
+        // block cg of every k quarter: rows 4(cg&1).. of the units 4(2s'+(cg>>1))+q
+        const int cg = (lane >> 2) & 3, t = lane & 3;
+        const uint4 *src = Au + (int64_t)(row0 + 4 * (cg & 1) + t) * ROW_UNITS + 4 * (cg >> 1) + q;
+#pragma unroll
+        for (int s2 = 0; s2 < A_REGS; ++s2) a[s2] = src[s2 * 8];
+    } else {
+        // panel rows: lanes 8..15 of every 16 repeat rows 0..7, their results are not stored
         const uint4 *src = Au + (int64_t)(row0 + (n & 7)) * ROW_UNITS + q;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
@@ -1049,10 +1130,33 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
         r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)w_);
         return r;
     };
+    // 4x4 blocks: both row halves of 16 columns, partial over the k quarters
+    auto compute_blocks = [&](const Oper &o, f32x4_t &lo, f32x4_t &hi) {
+        lo = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        hi = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if constexpr (BLOCKS) {
+#pragma unroll
+            for (int s2 = 0; s2 < A_REGS; ++s2) {
+                {
+                    const uint4 b = permute4(to_operand_from, o.b[2 * s2].x, o.b[2 * s2].y, o.b[2 * s2].z, o.b[2 * s2].w);
+                    mfma_blocks_unit<0>(a[s2], b, lo, hi);
+                    __builtin_amdgcn_sched_group_barrier(0x080, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+                }
+                {
+                    const uint4 b = permute4(to_operand_from, o.b[2 * s2 + 1].x, o.b[2 * s2 + 1].y, o.b[2 * s2 + 1].z,
+                                             o.b[2 * s2 + 1].w);
+                    mfma_blocks_unit<2>(a[s2], b, lo, hi);
+                    __builtin_amdgcn_sched_group_barrier(0x080, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+                }
+            }
+        }
+    };
     auto compute = [&](const Oper &o) {
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
+        for (int s = 0; s < (BLOCKS ? 0 : STEPS); ++s) {
             const uint4 b = permute4(to_operand_from, o.b[s].x, o.b[s].y, o.b[s].z, o.b[s].w);
             if constexpr (DT == DT_BF16) {
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, b),
@@ -1082,15 +1186,37 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
     // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
     auto compute_store_pair = [&](const Oper &o0, const Oper &o1, int g0) {
         if (g0 >= end) return;                                   // wave-uniform
-        const f32x4_t acc0 = compute(o0);
-        const f32x4_t acc1 = compute(o1);                        // columns clamped past the end: computed, not stored
-        // result lane (n,q) holds entries 4q.. of its group for row n&7: lanes with n < 8 keep
-        // the first group's, lanes with n >= 8 the second group's; memory lane l wants row l>>3,
-        // entries g0+4(l&7)..
-        // (element values first: a bit cast applied to a vector element expression reads element 0)
-        const bool second = (n & 8) != 0;
-        const float r0 = second ? acc1[0] : acc0[0], r1 = second ? acc1[1] : acc0[1];
-        const float r2 = second ? acc1[2] : acc0[2], r3 = second ? acc1[3] : acc0[3];
+        float r0, r1, r2, r3;
+        if constexpr (BLOCKS) {
+            f32x4_t lo0, hi0, lo1, hi1;
+            compute_blocks(o0, lo0, hi0);
+            compute_blocks(o1, lo1, hi1);                        // columns clamped past the end: computed, not stored
+            // register i of lane (q,cg,j): row i (lo) / 4+i (hi), column 4cg+j of its group, partial
+            // over q = (bit 5, bit 4) of the lane.  First swap: the two lane halves add up, the lower
+            // keeps rows 0..3, the upper rows 4..7; second swap: the 16-lane rows add up, even rows
+            // keep the first group, odd rows the second.  Lane (b5,b4,cg,j), register i is then
+            // (row 4 b5 + i, column 16 b4 + 4 cg + j of the pair); the transpose makes it
+            // (row 4 b5 + j, columns 16 b4 + 4 cg + i).
+            float f[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float g_first = swap32_add(lo0[i], hi0[i]);
+                const float g_second = swap32_add(lo1[i], hi1[i]);
+                f[i] = swap16_add(g_first, g_second);
+            }
+            quad_transpose(f, lane);
+            r0 = f[0]; r1 = f[1]; r2 = f[2]; r3 = f[3];
+        } else {
+            const f32x4_t acc0 = compute(o0);
+            const f32x4_t acc1 = compute(o1);                    // columns clamped past the end: computed, not stored
+            // result lane (n,q) holds entries 4q.. of its group for row n&7: lanes with n < 8 keep
+            // the first group's, lanes with n >= 8 the second group's; memory lane l wants row l>>3,
+            // entries g0+4(l&7)..
+            // (element values first: a bit cast applied to a vector element expression reads element 0)
+            const bool second = (n & 8) != 0;
+            r0 = second ? acc1[0] : acc0[0]; r1 = second ? acc1[1] : acc0[1];
+            r2 = second ? acc1[2] : acc0[2]; r3 = second ? acc1[3] : acc0[3];
+        }
         const uint4 m = permute4(to_memory_from, __builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1),
                                  __builtin_bit_cast(uint32_t, r2), __builtin_bit_cast(uint32_t, r3));
         const float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
