@@ -62,6 +62,7 @@ __device__ __forceinline__ int sum16(int v) {
 // stops early when on_tile returns false (it must return the same in all 16 lanes).
 // Returns false in a lane whose row is not strictly increasing in column.
 struct __attribute__((packed, aligned(4))) I4u { int x, y, z, w; };
+struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
 
 template <class F>
 __device__ __forceinline__ bool walk_strip(const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col, int M,
@@ -875,17 +876,253 @@ __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void
     }
 }
 
+// ---- windows of four tiles ---------------------------------------------------------
+// A wavefront that walks its tiles one after the other spends its life waiting: a launch
+// of this path lasts a dozen microseconds, a dependent memory round trip about one, and
+// the walk chains descriptor -> operands -> result for every tile.  So the unit of work is
+// a WINDOW of TILE_WINDOW consecutive descriptors of one strip, handled as a batch with
+// two round trips: (1) the window record, one dword per lane; (2) everything else at once
+// -- the A panel, the B rows of all its tiles, and the S values and column indices.
+//
+// S and P are not accessed per (row, tile): the entries of row r inside the window's
+// tiles are consecutive in the CSR arrays (the tiles are consecutive present tiles of the
+// strip, so nothing of the row lies between them), cnt[r] entries from p0[r].  Four
+// lanes per row read and write them 16 bytes at a time whatever the fill of the tiles
+// (the last lane of a row moves its four entries back so that they end with the row's
+// run: some entries are written twice with the same value, none is written in parts).
+// The products come from the matrix cores in result layout, pass through LDS (written
+// by columns of 16 rows, 16 bytes per lane) and are picked up per entry: its column says
+// which tile and which column of the tile.  Per window of four tiles with 92 entries
+// each: 20 memory instructions instead of 56.
+//
+// A window whose descriptors are not plain aligned tiles of one strip (a strip ends
+// inside it, union tiles) is flagged by the plan and walked tile by tile (tile_wave).
+constexpr int TILE_WINDOW = 4;
+constexpr int WIN_PITCH = 20;                 // floats per result column in LDS: 16 rows, padded, 16-byte aligned
+constexpr int WIN_LDS_FLOATS = TILE_WINDOW * 16 * WIN_PITCH;
+
+struct alignas(16) TileWindow {               // lane l < 48 loads dword l
+    int32_t arow[16];    // row of A for strip row r (row 0 where the strip has no such row: then cnt is 0)
+    int32_t p0[16];      // CSR position of row r's first entry inside the window
+    uint16_t cnt[16];    // entries of row r inside the window (consecutive from p0)
+    int32_t tj[TILE_WINDOW];   // tile columns, -1 where the window has fewer tiles
+    int32_t flags;       // != 0: walk the window tile by tile
+    int32_t maxcnt;      // largest cnt
+    int32_t pad[2];
+};
+static_assert(sizeof(TileWindow) == 192, "TileWindow layout");
+
+// plan: one thread per (window, strip row)
+__global__ __launch_bounds__(256) void k_tile_windows(const int32_t *__restrict__ vrows, int M, int64_t nnz,
+                                                      const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                      int64_t union_lo, int64_t union_hi,
+                                                      TileWindow *__restrict__ win, int64_t n_win) {
+    const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t w = slot >> 4;
+    const int r = (int)(slot & 15);
+    if (w >= n_win) return;                   // groups of 16 lanes leave together
+    const int64_t t0 = w * TILE_WINDOW;
+    const int n = (int)(n_tiles - t0 < TILE_WINDOW ? n_tiles - t0 : TILE_WINDOW);
+    const int4 h0 = *reinterpret_cast<const int4 *>(tiles + t0);          // strip, tj, pad[0], pad[1]
+    // the 16-byte accesses of the batch need four entries to exist
+    bool mixed = (t0 < union_hi && t0 + n > union_lo) || nnz < 4;
+    int tj[TILE_WINDOW];
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) {
+        tj[k] = -1;
+        if (k < n) {
+            const int4 h = *reinterpret_cast<const int4 *>(tiles + t0 + k);
+            tj[k] = h.y;
+            mixed |= h.x != h0.x;
+        }
+    }
+    const int strip = h0.x;
+    const int64_t row = strip >= GATHERED_BASE ? (int64_t)vrows[(int64_t)(strip - GATHERED_BASE) * 16 + r]
+                                               : (int64_t)strip * 16 + r;
+    const bool valid = row >= 0 && row < M;
+    const TileDesc *last = tiles + t0 + n - 1;
+    const int p0 = tiles[t0].off[r];
+    int cnt = valid && !mixed ? last->off[r] + __builtin_popcount((unsigned int)last->mask[r]) - p0 : 0;
+    cnt = cnt < 0 ? 0 : (cnt > 16 * TILE_WINDOW ? 16 * TILE_WINDOW : cnt);
+    const int mx = max16(cnt);
+    TileWindow *o = win + w;
+    o->arow[r] = valid ? (int32_t)row : 0;
+    o->p0[r] = p0;
+    o->cnt[r] = (uint16_t)cnt;
+    if (r == 0) {
+#pragma unroll
+        for (int k = 0; k < TILE_WINDOW; ++k) o->tj[k] = tj[k];
+        o->flags = mixed ? 1 : 0;
+        o->maxcnt = mx;
+        o->pad[0] = o->pad[1] = 0;
+    }
+}
+
+// window w on the calling wavefront; lds: WIN_LDS_FLOATS floats of its own
+template <int DT, int STEPS>
+__device__ __forceinline__ void tile_window_wave(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                                 const int32_t *__restrict__ vrows,
+                                                 const int32_t *__restrict__ tile_cols,
+                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                 const TileWindow *__restrict__ win, int64_t n_win,
+                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                 float *__restrict__ P, int64_t nnz, int64_t w, float *lds) {
+    if (w >= n_win) return;
+    const int lane = lane_id();
+    if (win == nullptr) {                                 // the plan chose the tile-by-tile walk for this matrix
+        tile_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, TILE_WINDOW, sval, P, w);
+        return;
+    }
+    const int32_t *rec = reinterpret_cast<const int32_t *>(win + w);
+    const int dw = rec[lane < 48 ? lane : 47];
+    if (__builtin_amdgcn_readlane(dw, 44) != 0) {
+        tile_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, TILE_WINDOW, sval, P, w);
+        return;
+    }
+    const int maxcnt = __builtin_amdgcn_readlane(dw, 45);
+    if (maxcnt <= 0) return;
+    const int r16 = lane & 15, q = lane >> 4;        // operand / result layout
+    const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: four neighbouring lanes on 64 bytes of a row
+    const int to_operand_from = (4 * r16 + q) << 2;
+    constexpr uint32_t ROW_UNITS = STEPS * 4;
+    const uint4 *__restrict__ Au = (const uint4 *)A;
+    const uint4 *__restrict__ Bu = (const uint4 *)B;
+    auto to_operand = [&](const uint4 &v) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.w);
+        return r;
+    };
+    int tj[TILE_WINDOW];
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) tj[k] = __builtin_amdgcn_readlane(dw, 40 + k);
+    // the row of the S/P accesses of this lane: strip row lane>>2, its entries 4(lane&3)+16m.. of the window
+    const int p0 = __shfl(dw, 16 + lrow, WAVE);
+    const int cw = __shfl(dw, 32 + (lrow >> 1), WAVE);
+    const int cnt = (lrow & 1) ? (int)((unsigned int)cw >> 16) : (cw & 0xFFFF);
+    const int64_t arow = __shfl(dw, lrow, WAVE);
+    auto entry_pos = [&](int m) {
+        int ws = 4 * lunit + 16 * m;
+        ws = ws < cnt - 4 ? ws : cnt - 4;
+        ws = ws < 0 ? 0 : ws;
+        const int64_t pos = (int64_t)p0 + ws;
+        return pos < nnz - 4 ? pos : nnz - 4;            // only rows of fewer than four entries can get here
+    };
+    // ---- second round trip: everything at once ----------------------------------------
+    uint4 a_mem[STEPS];
+    {
+        const uint4 *src = Au + arow * ROW_UNITS + lunit;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) a_mem[s] = src[s * 4];
+    }
+    auto load_b = [&](int k, uint4 (&dst)[STEPS]) {
+        int64_t brow = (int64_t)(tj[k] < 0 ? 0 : tj[k]) * 16 + lrow;
+        brow = brow < N ? brow : N - 1;                   // columns past N are in no row's entries
+        const uint4 *src = Bu + brow * ROW_UNITS + lunit;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) dst[s] = src[s * 4];
+    };
+    constexpr bool ALL_B = STEPS <= 4;                    // rows of up to 256 bytes: the B rows of all four tiles in flight
+    uint4 b[ALL_B ? TILE_WINDOW : 2][STEPS];
+    if constexpr (ALL_B) {
+#pragma unroll
+        for (int k = 0; k < TILE_WINDOW; ++k) load_b(k, b[k]);
+    } else {
+        load_b(0, b[0]);
+    }
+    const int iters = (maxcnt + 15) >> 4;                 // wave-uniform, 1..4
+    I4u c_pre[2];
+    F4u s_pre[2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+        const int64_t pos = entry_pos(m < iters ? m : 0);
+        c_pre[m] = *reinterpret_cast<const I4u *>(col + pos);
+        s_pre[m] = *reinterpret_cast<const F4u *>(sval + pos);
+    }
+    // ---- products of every tile into LDS ------------------------------------------------
+    uint4 a[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) a[s] = to_operand(a_mem[s]);
+    auto product = [&](const uint4 (&bt)[STEPS], int k) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const uint4 bo = to_operand(bt[s]);
+            if constexpr (DT == DT_BF16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
+                                                              __builtin_bit_cast(bf16x8_t, bo), acc, 0, 0, 0);
+            } else if constexpr (DT == DT_F16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a[s]),
+                                                             __builtin_bit_cast(half8_t, bo), acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
+                                                           __builtin_bit_cast(float, bo.x), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].y),
+                                                           __builtin_bit_cast(float, bo.y), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].z),
+                                                           __builtin_bit_cast(float, bo.z), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].w),
+                                                           __builtin_bit_cast(float, bo.w), acc, 0, 0, 0);
+            }
+        }
+        // result register i of lane (r16, q) is row 4q+i, column r16 of tile k
+        *reinterpret_cast<f32x4_t *>(lds + (k * 16 + r16) * WIN_PITCH + 4 * q) = acc;
+    };
+    if constexpr (ALL_B) {
+#pragma unroll
+        for (int k = 0; k < TILE_WINDOW; ++k)
+            if (tj[k] >= 0) product(b[k], k);             // wave-uniform
+    } else {
+#pragma unroll
+        for (int k = 0; k < TILE_WINDOW; ++k) {
+            if (tj[k] < 0) break;                         // wave-uniform
+            if (k + 1 < TILE_WINDOW && tj[k + 1 < TILE_WINDOW ? k + 1 : k] >= 0) load_b(k + 1, b[(k + 1) & 1]);
+            product(b[k & 1], k);
+        }
+    }
+    wave_lds_order();
+    // ---- entries: four per lane, 16 per row and iteration -----------------------------------
+    const int t1 = tj[1], t2 = tj[2], t3 = tj[3];
+    auto pick = [&](int c) {
+        const int tc = c >> 4;
+        const int k = (tc == t1 ? 1 : 0) + (tc == t2 ? 2 : 0) + (tc == t3 ? 3 : 0);
+        return lds[(k * 16 + (c & 15)) * WIN_PITCH + lrow];
+    };
+    for (int m = 0; m < iters; ++m) {
+        I4u c4;
+        F4u s4;
+        if (m < 2) { c4 = c_pre[m]; s4 = s_pre[m]; }
+        else {
+            const int64_t pos = entry_pos(m);
+            c4 = *reinterpret_cast<const I4u *>(col + pos);
+            s4 = *reinterpret_cast<const F4u *>(sval + pos);
+        }
+        const bool active = cnt >= 4 && 4 * lunit + 16 * m < cnt;
+        const F4u out{pick(c4.x) * s4.x, pick(c4.y) * s4.y, pick(c4.z) * s4.z, pick(c4.w) * s4.w};
+        if (active) *reinterpret_cast<F4u *>(P + entry_pos(m)) = out;
+    }
+    // rows with one to three entries in the window: entry by entry
+    if (cnt > 0 && cnt < 4 && lunit == 0) {
+        for (int e = 0; e < cnt; ++e) P[(int64_t)p0 + e] = pick(col[(int64_t)p0 + e]) * sval[(int64_t)p0 + e];
+    }
+    wave_lds_order();                                     // the next window of this wave reuses the buffer
+}
+
 template <int DT, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
                                                 const int32_t *__restrict__ vrows,
                                                 const int32_t *__restrict__ tile_cols,
                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
-                                                int tiles_per_wave, const float *__restrict__ sval,
-                                                float *__restrict__ P, int64_t nblocks) {
+                                                const TileWindow *__restrict__ win, int64_t n_win,
+                                                const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                float *__restrict__ P, int64_t nnz, int64_t nblocks) {
+    __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
-    tile_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, tiles_per_wave, sval, P,
-                         blk * WAVES_PER_BLOCK + wave_in_block());
+    tile_window_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
+                                blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()]);
 }
 
 // AUTO in one launch when a matrix has tiles and rows: logical blocks are dealt out
@@ -904,13 +1141,16 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
                                                       const int32_t *__restrict__ vrows,
                                                       const int32_t *__restrict__ tile_cols,
                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
-                                                      int tiles_per_wave, int64_t tile_blocks, int64_t nblocks) {
+                                                      const TileWindow *__restrict__ win, int64_t n_win, int64_t nnz,
+                                                      int64_t tile_blocks, int64_t nblocks) {
+    __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int64_t tiles_before = blk * tile_blocks / nblocks;
     if (((blk + 1) * tile_blocks / nblocks) != tiles_before) {
-        tile_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, tiles_per_wave, sval, P,
-                                   tiles_before * WAVES_PER_BLOCK + wave_in_block());
+        tile_window_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
+                                          tiles_before * WAVES_PER_BLOCK + wave_in_block(),
+                                          win_lds[wave_in_block()]);
         return;
     }
     const int64_t rb = blk - tiles_before, rest = nblocks - tile_blocks;
@@ -987,8 +1227,6 @@ __global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A
 // groups of a pair out to the lanes, a 4x4 transpose inside every quad (two DPP stages)
 // turns (register = row, lane = column) into (lane = row, register = column): four
 // consecutive entries of a row per lane, which then move to the memory layout as above.
-struct __attribute__((packed, aligned(4))) F4u { float x, y, z, w; };
-
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 
 template <int ABID>

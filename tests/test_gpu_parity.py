@@ -866,3 +866,42 @@ def test_union_strips(engine_factory, monkeypatch, K, dtype):
     off, st0 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
     assert st0.mfma_tiles == 0
     assert_parity(off, rowptr, col, val, A, B, what="union strips off")
+
+
+@pytest.mark.parametrize("fill_limit", ["0", "100000"])
+@pytest.mark.parametrize("K,dtype", [(32, capi.F32), (64, capi.F32), (128, capi.BF16), (256, capi.F32), (512, capi.BF16)])
+def test_tile_windows_and_tile_walk_agree_with_the_oracle(engine_factory, monkeypatch, fill_limit, K, dtype):
+    """The tile kernels take four consecutive tiles of a strip either as one batch (the
+    entries of a row inside the window read and written as runs; SDDMM_WINDOW_FILL above
+    the fill of the tiles) or tile by tile (below it).  Both on strips whose rows hold
+    0, 1, 2, 3, 4, 5 and many entries per window, on a strip count that is not a multiple
+    of anything, with the last window of a strip shorter than four tiles."""
+    monkeypatch.setenv("SDDMM_WINDOW_FILL", fill_limit)
+    rng = np.random.default_rng(4100 + K)
+    M, N = 16 * 9 + 3, 16 * 41 + 7
+    dense = np.zeros((M, N), bool)
+    for s in range(M // 16 + 1):
+        r0 = 16 * s
+        tiles = np.sort(rng.choice(N // 16, int(rng.integers(1, 15)), replace=False))
+        for tj in tiles:
+            blk = rng.random((16, 16)) < rng.choice([0.08, 0.3, 0.9, 1.0])
+            dense[r0:r0 + 16, 16 * tj:16 * tj + 16][: M - r0] |= blk[: M - r0]
+        # rows of the strip with very few entries, and empty ones
+        for rr, keep in ((1, 1), (2, 2), (3, 3), (5, 4), (6, 5), (7, 0)):
+            if r0 + rr < M:
+                c = np.nonzero(dense[r0 + rr])[0]
+                dense[r0 + rr] = False
+                dense[r0 + rr, c[:keep]] = True
+    r, c = np.nonzero(dense)
+    v = rng.uniform(-1, 1, len(r)).astype(f32)
+    rowptr, col, val = O.csr_from_triplets(M, r.astype(np.int32), c.astype(np.int32), v)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == capi.BF16:
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K)
+    else:
+        Ab, Bb = A, B
+    got, st = run_csr(engine_factory, rowptr, col, val, Ab, Bb, N, capi.MFMA_TILE, dtype)
+    assert st.nnz_mfma == len(col) and st.mfma_tiles > 0
+    assert_parity(got, rowptr, col, val, A, B, what="tiles K=%d limit %s" % (K, fill_limit))
