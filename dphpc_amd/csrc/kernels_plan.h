@@ -75,6 +75,33 @@ __device__ __forceinline__ unsigned int wave_max_u32(unsigned int v) {
     return v;
 }
 
+// What a plan clears before its classifiers run, in one launch (a fill through the
+// runtime is a launch of its own for every region): the row-ownership bytes and every
+// counter except what validation measured (non-empty rows, longest row).  rows_only: just
+// the row classes and the item total, for the second count after the gathered strips.
+__global__ __launch_bounds__(256) void k_plan_reset(unsigned char *__restrict__ owner, int64_t owner_bytes,
+                                                    DevCounters *pc, int rows_only) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (!rows_only) {
+        // 16 bytes per thread (the array is 256-byte aligned and padded to 64 bytes past the rows)
+        const int64_t at = i * 16;
+        if (at + 16 <= owner_bytes) *reinterpret_cast<uint4 *>(owner + at) = make_uint4(0u, 0u, 0u, 0u);
+        else for (int64_t q = at; q < owner_bytes; ++q) owner[q] = 0;
+    }
+    if (blockIdx.x == 0) {
+        const int first = K_ROWS_SHORT, last = rows_only ? K_NNZ_LONG : K_NNZ_PANELS;
+        for (int k = first; k <= last; ++k)
+            for (int sl = threadIdx.x; sl < SPREAD; sl += blockDim.x) pc->k[k][sl] = 0ull;
+        if (threadIdx.x == 0) {
+            pc->n_items = 0ull;
+            if (!rows_only) {
+                pc->tiles_scanned = 0ull; pc->panel_items = 0ull; pc->n_candidates = 0ull; pc->utiles_scanned = 0ull;
+                pc->pad3 = 0ull;
+            }
+        }
+    }
+}
+
 // rowptr[0]==0, rowptr[M]==nnz, non-decreasing; also counts non-empty rows and the
 // longest row.  One lane per row, one set of atomics per workgroup.
 __global__ __launch_bounds__(256) void k_check_rowptr(const int32_t *__restrict__ rowptr, int M,

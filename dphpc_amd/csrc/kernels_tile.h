@@ -1130,8 +1130,11 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
 // so that every XCD gets its share of each.  Kernels of one stream run one after
 // the other; two short launches leave the chip half idle twice, one launch does not.
 // L must be the full-K, 32-bit-offset layout of a row of STEPS * 64 bytes.
+#ifndef SDDMM_FUSED_WAVES
+#define SDDMM_FUSED_WAVES 6
+#endif
 template <class L, int STEPS>
-__global__ __launch_bounds__(BLOCK) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
+__global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                       const int32_t *__restrict__ rowptr,
                                                       const unsigned char *__restrict__ owner,
                                                       const int32_t *__restrict__ col,

@@ -94,6 +94,10 @@ struct sddmm_ctx {
     // row ownership (one byte per row: 0 row kernels, 1 dense tiles, 2 row panels, 3 gathered strips, 4 union strips)
     unsigned char *d_owner = nullptr;
     int64_t owner_cap = 0;
+    // every work array of the plan whose size follows from the number of rows lives in one
+    // allocation (a first plan then pays for one hipMalloc instead of a dozen)
+    char *d_arena = nullptr;
+    int64_t arena_rows = -1;
     bool owner_active = false;
     // row-panel path
     unsigned int *d_panel_counts = nullptr, *d_panel_off = nullptr;
@@ -174,6 +178,66 @@ void dfree(T *&p) {
     p = nullptr;
 }
 
+// Views into the plan arena: nothing here is freed on its own.
+void release_arena(sddmm_ctx *c) {
+    dfree(c->d_arena);
+    c->arena_rows = -1;
+    c->d_owner = nullptr;
+    c->d_strip_ntiles = c->d_strip_off = c->d_ustrip_ntiles = c->d_ustrip_off = nullptr;
+    c->d_panel_counts = c->d_panel_off = c->d_vstrip_ntiles = c->d_vstrip_off = nullptr;
+    c->d_cand_keys = c->d_sorted_keys = nullptr;
+    c->d_vrows = nullptr;
+    c->d_block_sums = nullptr;
+    c->owner_cap = c->strips_cap = c->ustrips_cap = c->panels_cap = c->cand_cap = c->vstrips_cap = 0;
+    c->block_sums_cap = 0;
+}
+
+int ensure_arena(sddmm_ctx *c) {
+    const int64_t M = c->sM;
+    if (c->d_arena && c->arena_rows == M) return SDDMM_OK;
+    release_arena(c);
+    const int64_t n_strips = (M + 15) / 16, n_panels = M / 8 + 1, n_sums = M / 1024 + 2;
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        const size_t here = at;
+        at += (bytes + 255) & ~(size_t)255;
+        return here;
+    };
+    const size_t o_owner = take((size_t)M + 64);
+    const size_t o_strip_n = take((size_t)n_strips * 4), o_strip_o = take((size_t)n_strips * 4);
+    const size_t o_ustrip_n = take((size_t)n_strips * 4), o_ustrip_o = take((size_t)n_strips * 4);
+    const size_t o_vstrip_n = take((size_t)n_strips * 4), o_vstrip_o = take((size_t)n_strips * 4);
+    const size_t o_vrows = take((size_t)n_strips * 16 * 4);
+    const size_t o_panel_n = take((size_t)n_panels * 4), o_panel_o = take((size_t)n_panels * 4);
+    const size_t o_keys = take((size_t)(M + 1) * 8), o_sorted = take((size_t)(M + 1) * 8);
+    const size_t o_sums = take((size_t)n_sums * 4);
+    ALLOC_TRY(c, c->d_arena, at);
+    char *b = c->d_arena;
+    c->d_owner = (unsigned char *)(b + o_owner);
+    c->d_strip_ntiles = (unsigned int *)(b + o_strip_n); c->d_strip_off = (unsigned int *)(b + o_strip_o);
+    c->d_ustrip_ntiles = (unsigned int *)(b + o_ustrip_n); c->d_ustrip_off = (unsigned int *)(b + o_ustrip_o);
+    c->d_vstrip_ntiles = (unsigned int *)(b + o_vstrip_n); c->d_vstrip_off = (unsigned int *)(b + o_vstrip_o);
+    c->d_vrows = (int32_t *)(b + o_vrows);
+    c->d_panel_counts = (unsigned int *)(b + o_panel_n); c->d_panel_off = (unsigned int *)(b + o_panel_o);
+    c->d_cand_keys = (unsigned long long *)(b + o_keys); c->d_sorted_keys = (unsigned long long *)(b + o_sorted);
+    c->d_block_sums = (unsigned int *)(b + o_sums);
+    c->owner_cap = M + 64;
+    c->strips_cap = c->ustrips_cap = c->vstrips_cap = n_strips;
+    c->panels_cap = n_panels;
+    c->cand_cap = M + 1;
+    c->block_sums_cap = n_sums;
+    c->arena_rows = M;
+    return SDDMM_OK;
+}
+
+// an arena view turned out too small: the sizes above are upper bounds, so this is a bug
+#define ARENA_HOLDS(c, need, cap, what)                                                             \
+    do {                                                                                            \
+        if ((int64_t)(need) > (int64_t)(cap))                                                       \
+            return fail((c), SDDMM_ERR_HIP, "internal: plan arena too small for %s (%lld > %lld)", what, \
+                        (long long)(need), (long long)(cap));                                       \
+    } while (0)
+
 void release_dense(sddmm_ctx *c) {
     if (c->own_dense) { dfree(c->dA); dfree(c->dB); }
     c->dA = c->dB = nullptr;
@@ -189,22 +253,15 @@ void release_sparse(sddmm_ctx *c) {
     if (c->own_rowidx) dfree(c->d_rowidx);
     dfree(c->dP);
     dfree(c->d_items);
-    dfree(c->d_block_sums);
-    dfree(c->d_strip_ntiles);
-    dfree(c->d_strip_off);
     dfree(c->d_tiles);
     dfree(c->d_tile_cols);
     dfree(c->d_windows);
     c->n_windows = c->windows_cap = 0;
-    dfree(c->d_ustrip_ntiles); dfree(c->d_ustrip_off);
     c->ustrips_cap = 0;
-    dfree(c->d_cand_keys); dfree(c->d_sorted_keys);
-    dfree(c->d_vrows); dfree(c->d_sort_tmp); dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off);
+    dfree(c->d_sort_tmp);
+    release_arena(c);
     c->sort_tmp_bytes = 0;
     c->cand_cap = c->vstrips_cap = c->n_cand = c->n_vstrips = 0;
-    dfree(c->d_owner);
-    dfree(c->d_panel_counts);
-    dfree(c->d_panel_off);
     dfree(c->d_panel_items);
     dfree(c->d_fused_items);
     c->n_fused_items = c->fused_items_cap = 0;
@@ -415,17 +472,15 @@ void launch_auto(sddmm_ctx *c) {
 // Row classifier: statistics, then the item list of the wave-per-segment kernel.
 // Row classes and work items of the rows nobody owns, in two halves around a read-back of the
 // counters: the count (launch only; it may be launched again after more rows found an owner) ...
-int classify_rows_count(sddmm_ctx *c) {
+int classify_rows_count(sddmm_ctx *c, bool again = false) {
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
-    if (nb > c->block_sums_cap) {
-        dfree(c->d_block_sums);
-        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
-        c->block_sums_cap = nb;
+    ARENA_HOLDS(c, nb, c->block_sums_cap, "block sums");
+    // the first count of a plan finds its counters cleared (begin_ownership); a second one keeps what
+    // validation and the ownership classifiers measured and clears the row classes
+    if (again) {
+        SDDMM_LAUNCH(c, k_plan_reset, 1, 256, c->d_owner, (int64_t)0, c->d_pc, 1);
+        LAUNCH_CHECK(c);
     }
-    // keep what validation and the ownership classifiers measured, clear the row classes
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
-                              sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     if (nb > 0) {
         const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr, owner,
@@ -465,11 +520,7 @@ int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t
         return SDDMM_OK;
     }
     const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
-    if (nb > c->block_sums_cap) {
-        dfree(c->d_block_sums);
-        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
-        c->block_sums_cap = nb;
-    }
+    ARENA_HOLDS(c, nb, c->block_sums_cap, "block sums");
     SDDMM_LAUNCH(c, k_scan_sums, nb, SCAN_BLOCK, in, n, c->d_block_sums);
     SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb, d_total);
     SDDMM_LAUNCH(c, k_scan_apply, nb, SCAN_BLOCK, in, n,
@@ -481,15 +532,12 @@ int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t
 // Clears the row-ownership bytes and the tile / panel counters before the classifiers run.
 int begin_ownership(sddmm_ctx *c) {
     const int64_t bytes = (int64_t)c->sM + 64;
-    if (bytes > c->owner_cap) {
-        dfree(c->d_owner);
-        ALLOC_TRY(c, c->d_owner, (size_t)bytes);
-        c->owner_cap = bytes;
-    }
-    HIP_TRY(c, hipMemsetAsync(c->d_owner, 0, (size_t)bytes, c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_TILES][0], 0,
-                              sizeof(unsigned long long) * SPREAD * (K_NNZ_PANELS - K_TILES + 1), c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->tiles_scanned, 0, 5 * sizeof(unsigned long long), c->stream));
+    const int arc = ensure_arena(c);
+    if (arc) return arc;
+    ARENA_HOLDS(c, bytes, c->owner_cap, "row owners");
+    // one launch clears the owners and every counter of the classifiers, the row classes included
+    SDDMM_LAUNCH(c, k_plan_reset, grid_for((bytes + 15) / 16, 256), 256, c->d_owner, bytes, c->d_pc, 0);
+    LAUNCH_CHECK(c);
     c->owner_active = true;
     c->tiles_active = false;
     c->n_tiles = c->nnz_tiles = c->n_tiles_natural = c->n_tiles_union = c->nnz_tiles_union = 0;
@@ -518,13 +566,7 @@ bool tile_path_applies(sddmm_ctx *c) {
 int plan_tiles_count(sddmm_ctx *c, int min_fill) {
     if (!tile_path_applies(c)) return SDDMM_OK;
     const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
-    if (n_strips > c->strips_cap) {
-        dfree(c->d_strip_ntiles);
-        dfree(c->d_strip_off);
-        ALLOC_TRY(c, c->d_strip_ntiles, (size_t)n_strips * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_strip_off, (size_t)n_strips * sizeof(unsigned int));
-        c->strips_cap = n_strips;
-    }
+    ARENA_HOLDS(c, n_strips, c->strips_cap, "strips");
     const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
     SDDMM_LAUNCH(c, k_strip_count, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                        c->d_col, c->sM, n_strips, min_fill, c->d_strip_ntiles, c->d_owner, c->d_pc);
@@ -552,13 +594,7 @@ int take_tile_counts(sddmm_ctx *c) {
 int plan_union_count(sddmm_ctx *c, int min_fill) {
     if (c->tile_steps == 0) return SDDMM_OK;
     const int64_t n_strips = ((int64_t)c->sM + 15) / 16;
-    if (n_strips > c->ustrips_cap) {
-        dfree(c->d_ustrip_ntiles);
-        dfree(c->d_ustrip_off);
-        ALLOC_TRY(c, c->d_ustrip_ntiles, (size_t)n_strips * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_ustrip_off, (size_t)n_strips * sizeof(unsigned int));
-        c->ustrips_cap = n_strips;
-    }
+    ARENA_HOLDS(c, n_strips, c->ustrips_cap, "union strips");
     const unsigned strip_grid = (unsigned)((n_strips + STRIPS_PER_BLOCK - 1) / STRIPS_PER_BLOCK);
     SDDMM_LAUNCH(c, k_union_count, strip_grid, WAVE * STRIPS_PER_BLOCK, c->d_rowptr,
                        c->d_col, c->sM, n_strips, min_fill, c->d_owner, c->d_ustrip_ntiles, c->d_pc);
@@ -572,12 +608,7 @@ int plan_union_count(sddmm_ctx *c, int min_fill) {
 int plan_gathered_candidates(sddmm_ctx *c, int min_len) {
     if (c->tile_steps == 0 || c->sM < 2) return SDDMM_OK;
     const int64_t M = c->sM;
-    if (M > c->cand_cap) {
-        dfree(c->d_cand_keys); dfree(c->d_sorted_keys);
-        ALLOC_TRY(c, c->d_cand_keys, (size_t)M * sizeof(unsigned long long));
-        ALLOC_TRY(c, c->d_sorted_keys, (size_t)M * sizeof(unsigned long long));
-        c->cand_cap = M;
-    }
+    ARENA_HOLDS(c, M, c->cand_cap, "candidate rows");
     SDDMM_LAUNCH(c, k_gather_candidates, ((M + 255) / 256), 256, c->d_rowptr,
                        c->d_col, c->sM, (const unsigned char *)c->d_owner, min_len, c->d_cand_keys,
                        &c->d_pc->n_candidates);
@@ -604,13 +635,7 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill, bool *launched) {
     HIP_TRY(c, rocprim::radix_sort_keys(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
                                         c->stream));
     c->n_vstrips = (c->n_cand + 15) / 16;
-    if (c->n_vstrips > c->vstrips_cap) {
-        dfree(c->d_vstrip_ntiles); dfree(c->d_vstrip_off); dfree(c->d_vrows);
-        ALLOC_TRY(c, c->d_vstrip_ntiles, (size_t)c->n_vstrips * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_vstrip_off, (size_t)c->n_vstrips * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_vrows, (size_t)c->n_vstrips * 16 * sizeof(int32_t));
-        c->vstrips_cap = c->n_vstrips;
-    }
+    ARENA_HOLDS(c, c->n_vstrips, c->vstrips_cap, "gathered strips");
     SDDMM_LAUNCH(c, k_gathered_count, c->n_vstrips, GATHERED_BLOCK, c->d_rowptr, c->d_col,
                        (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
                        c->d_vrows, c->d_owner, c->d_pc);
@@ -715,13 +740,7 @@ int plan_panels_flags(sddmm_ctx *c, int min_len, int pseg) {
     if (c->panel_mfma) min_len = std::max(min_len, 4);   // 16-byte S/P accesses stay inside a row
     const int64_t n_panels = (int64_t)c->sM / 8;
     if (n_panels == 0) return SDDMM_OK;
-    if (n_panels > c->panels_cap) {
-        dfree(c->d_panel_counts);
-        dfree(c->d_panel_off);
-        ALLOC_TRY(c, c->d_panel_counts, (size_t)n_panels * sizeof(unsigned int));
-        ALLOC_TRY(c, c->d_panel_off, (size_t)n_panels * sizeof(unsigned int));
-        c->panels_cap = n_panels;
-    }
+    ARENA_HOLDS(c, n_panels, c->panels_cap, "panels");
     SDDMM_LAUNCH(c, k_panel_flags, ((n_panels * WAVE + 255) / 256), 256,
                        c->d_rowptr, c->d_col, c->sM, n_panels, min_len, pseg, c->d_owner, c->d_panel_counts, c->d_pc);
     LAUNCH_CHECK(c);
@@ -971,7 +990,7 @@ int do_plan(sddmm_ctx *c, int strategy) {
                 if (rc) return rc;
                 if (launched) {
                     // gathered strips may have taken rows: classify again, one more read-back
-                    rc = classify_rows_count(c);
+                    rc = classify_rows_count(c, true);
                     if (rc) return rc;
                     rc = fetch_counters(c);
                     if (rc) return rc;
@@ -1366,11 +1385,9 @@ static int plan_fused_items(sddmm_ctx *c) {
     if (c->fused_items_valid) return SDDMM_OK;
     const int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
-    if (nb > c->block_sums_cap) {
-        dfree(c->d_block_sums);
-        ALLOC_TRY(c, c->d_block_sums, (size_t)nb * sizeof(unsigned int));
-        c->block_sums_cap = nb;
-    }
+    const int arc = ensure_arena(c);
+    if (arc) return arc;
+    ARENA_HOLDS(c, nb, c->block_sums_cap, "block sums");
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
                               sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
     HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
