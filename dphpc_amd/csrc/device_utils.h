@@ -110,6 +110,13 @@ struct UnitF32x4 {
         acc = __builtin_fmaf(a.w, b.w, acc);
         return acc;
     }
+    // acc[e] += p * (element e of b)
+    static __device__ __forceinline__ void axpy(float p, const T &b, float (&acc)[ELEMS]) {
+        acc[0] = __builtin_fmaf(p, b.x, acc[0]);
+        acc[1] = __builtin_fmaf(p, b.y, acc[1]);
+        acc[2] = __builtin_fmaf(p, b.z, acc[2]);
+        acc[3] = __builtin_fmaf(p, b.w, acc[3]);
+    }
 };
 struct UnitF32x1 {
     static constexpr int DT = DT_F32;
@@ -138,6 +145,12 @@ struct UnitBF16x8 {
         acc = __builtin_fmaf(hi(a.w), hi(b.w), acc);
         return acc;
     }
+    static __device__ __forceinline__ void axpy(float p, const T &b, float (&acc)[ELEMS]) {
+        acc[0] = __builtin_fmaf(p, lo(b.x), acc[0]); acc[1] = __builtin_fmaf(p, hi(b.x), acc[1]);
+        acc[2] = __builtin_fmaf(p, lo(b.y), acc[2]); acc[3] = __builtin_fmaf(p, hi(b.y), acc[3]);
+        acc[4] = __builtin_fmaf(p, lo(b.z), acc[4]); acc[5] = __builtin_fmaf(p, hi(b.z), acc[5]);
+        acc[6] = __builtin_fmaf(p, lo(b.w), acc[6]); acc[7] = __builtin_fmaf(p, hi(b.w), acc[7]);
+    }
 };
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -157,6 +170,22 @@ struct UnitF16x8 {
         acc = dot2(a.z, b.z, acc);
         acc = dot2(a.w, b.w, acc);
         return acc;
+    }
+    static __device__ __forceinline__ float lo(uint32_t w) {
+        const half2_t h = __builtin_bit_cast(half2_t, w);
+        const _Float16 e = h[0];
+        return (float)e;
+    }
+    static __device__ __forceinline__ float hi(uint32_t w) {
+        const half2_t h = __builtin_bit_cast(half2_t, w);
+        const _Float16 e = h[1];
+        return (float)e;
+    }
+    static __device__ __forceinline__ void axpy(float p, const T &b, float (&acc)[ELEMS]) {
+        acc[0] = __builtin_fmaf(p, lo(b.x), acc[0]); acc[1] = __builtin_fmaf(p, hi(b.x), acc[1]);
+        acc[2] = __builtin_fmaf(p, lo(b.y), acc[2]); acc[3] = __builtin_fmaf(p, hi(b.y), acc[3]);
+        acc[4] = __builtin_fmaf(p, lo(b.z), acc[4]); acc[5] = __builtin_fmaf(p, hi(b.z), acc[5]);
+        acc[6] = __builtin_fmaf(p, lo(b.w), acc[6]); acc[7] = __builtin_fmaf(p, hi(b.w), acc[7]);
     }
 };
 

@@ -6,7 +6,8 @@
 // The step that consumes an SDDMM result in the applications the reference names
 // (attention-like updates in graph learning); the reference itself stops at P.
 // The gathered B row of an entry is used twice while it sits in registers, so the
-// second product costs no memory traffic beyond the M x K output.
+// second product costs no memory traffic beyond the M x K output.  A and B may be fp32,
+// bf16 or fp16 (16-byte units of 4 or 8 elements); P and O are fp32.
 //
 // k_fusedmm: one wavefront per work item = entries [start,end) of one row (rows longer
 // than FUSED_ROW_MAX entries; shorter ones go to k_fusedmm_rows), in the lane layout
@@ -30,7 +31,8 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
                                                    float *__restrict__ O, const RowItem *__restrict__ items,
                                                    int64_t n_items, int64_t nblocks) {
     using U = typename L::U;
-    using T = typename U::T;                          // float4
+    using T = typename U::T;                          // 16 bytes: 4 fp32 or 8 bf16 / fp16
+    constexpr int E = U::ELEMS;
     using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
     using Off_t = typename C::O;
     constexpr int LPN = L::LPN, UPL = L::UPL, G = WAVE / LPN;
@@ -48,9 +50,11 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
     const int g = lane / LPN, j = lane & (LPN - 1);
     const Off_t rb = (Off_t)KU * (Off_t)sizeof(T);
     const typename C::Areg a = C::load_a(A, (Off_t)row * rb, j, KU);
-    T acc[UPL];
+    float acc[UPL][E];                                // the lane's units of the output row, fp32
 #pragma unroll
-    for (int i = 0; i < UPL; ++i) acc[i] = U::zero();
+    for (int i = 0; i < UPL; ++i)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[i][e] = 0.f;
     const int last = end - 1;
     for (int base = start; base < end; base += WAVE) {
         const int n = base + lane;
@@ -91,10 +95,12 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
                 p = live ? p : 0.f;
 #pragma unroll
                 for (int i = 0; i < UPL; ++i) {
-                    acc[i].x = live ? __builtin_fmaf(p, bf[q][i].x, acc[i].x) : acc[i].x;
-                    acc[i].y = live ? __builtin_fmaf(p, bf[q][i].y, acc[i].y) : acc[i].y;
-                    acc[i].z = live ? __builtin_fmaf(p, bf[q][i].z, acc[i].z) : acc[i].z;
-                    acc[i].w = live ? __builtin_fmaf(p, bf[q][i].w, acc[i].w) : acc[i].w;
+                    float next[E];
+#pragma unroll
+                    for (int e = 0; e < E; ++e) next[e] = acc[i][e];
+                    U::axpy(p, bf[q][i], next);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
                 }
                 if (j == t0 + q) out = p;
             }
@@ -107,27 +113,25 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
 #pragma unroll
     for (int off = LPN; off < WAVE; off <<= 1) {
 #pragma unroll
-        for (int i = 0; i < UPL; ++i) {
-            acc[i].x += __shfl_xor(acc[i].x, off, WAVE);
-            acc[i].y += __shfl_xor(acc[i].y, off, WAVE);
-            acc[i].z += __shfl_xor(acc[i].z, off, WAVE);
-            acc[i].w += __shfl_xor(acc[i].w, off, WAVE);
-        }
+        for (int i = 0; i < UPL; ++i)
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[i][e] += __shfl_xor(acc[i][e], off, WAVE);
     }
     if (g == 0) {
         const bool whole_row = start == rowptr[row] && end == rowptr[row + 1];
-        float *orow = O + (int64_t)row * KU * 4;
+        float *orow = O + (int64_t)row * KU * E;
 #pragma unroll
         for (int i = 0; i < UPL; ++i) {
             const int u = j + i * LPN;
             if (!C::unit_on(j, i, KU)) continue;
             if (whole_row) {
-                *reinterpret_cast<T *>(orow + 4 * u) = acc[i];
+#pragma unroll
+                for (int e = 0; e < E; e += 4)
+                    *reinterpret_cast<float4 *>(orow + E * u + e) =
+                        make_float4(acc[i][e], acc[i][e + 1], acc[i][e + 2], acc[i][e + 3]);
             } else {
-                atomicAdd(orow + 4 * u + 0, acc[i].x);
-                atomicAdd(orow + 4 * u + 1, acc[i].y);
-                atomicAdd(orow + 4 * u + 2, acc[i].z);
-                atomicAdd(orow + 4 * u + 3, acc[i].w);
+#pragma unroll
+                for (int e = 0; e < E; ++e) atomicAdd(orow + E * u + e, acc[i][e]);
             }
         }
     }
@@ -147,6 +151,7 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
                                                         float *__restrict__ O, int M, int max_len, int64_t nblocks) {
     using U = typename L::U;
     using T = typename U::T;
+    constexpr int E = U::ELEMS;
     using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
     using Off_t = typename C::O;
     constexpr int LPN = L::LPN, UPL = L::UPL, G = WAVE / LPN;
@@ -174,9 +179,11 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
     longest = __builtin_amdgcn_readfirstlane(longest);
     const Off_t rb = (Off_t)KU * (Off_t)sizeof(T);
     const typename C::Areg a = C::load_a(A, (Off_t)(row < M ? row : 0) * rb, j, KU);
-    T acc[UPL];
+    float acc[UPL][E];                                // the lane's units of the output row, fp32
 #pragma unroll
-    for (int i = 0; i < UPL; ++i) acc[i] = U::zero();
+    for (int i = 0; i < UPL; ++i)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[i][e] = 0.f;
     for (int t0 = 0; t0 < longest; t0 += LPN) {
         const int e = t0 + j;
         const bool has = e < len;
@@ -215,10 +222,12 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
                 p = live ? p : 0.f;
 #pragma unroll
                 for (int i = 0; i < UPL; ++i) {
-                    acc[i].x = live ? __builtin_fmaf(p, bf[q][i].x, acc[i].x) : acc[i].x;
-                    acc[i].y = live ? __builtin_fmaf(p, bf[q][i].y, acc[i].y) : acc[i].y;
-                    acc[i].z = live ? __builtin_fmaf(p, bf[q][i].z, acc[i].z) : acc[i].z;
-                    acc[i].w = live ? __builtin_fmaf(p, bf[q][i].w, acc[i].w) : acc[i].w;
+                    float next[E];
+#pragma unroll
+                    for (int e = 0; e < E; ++e) next[e] = acc[i][e];
+                    U::axpy(p, bf[q][i], next);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
                 }
                 if (j == q0 + q) out = p;
             }
@@ -226,11 +235,15 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
         if (has) P[at] = out;
     }
     if (mine) {
-        float *orow = O + row * KU * 4;
+        float *orow = O + row * KU * E;
 #pragma unroll
         for (int i = 0; i < UPL; ++i) {
             const int u = j + i * LPN;
-            if (C::unit_on(j, i, KU)) *reinterpret_cast<T *>(orow + 4 * u) = acc[i];
+            if (!C::unit_on(j, i, KU)) continue;
+#pragma unroll
+            for (int e = 0; e < E; e += 4)
+                *reinterpret_cast<float4 *>(orow + E * u + e) =
+                    make_float4(acc[i][e], acc[i][e + 1], acc[i][e + 2], acc[i][e + 3]);
         }
     }
 }

@@ -1423,8 +1423,10 @@ int sddmm_run_fused(sddmm_ctx *c) {
     int rc = check_ready(c);
     if (rc) return rc;
     const Shape s = shape_of(c);
-    if (c->dtype != SDDMM_F32 || s.unit != 0 || s.LPN == 0 || s.LPN > 8)
-        return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs fp32 operands with K a multiple of 4, K <= 256");
+    // 16-byte units, at most 8 lanes per entry and 32 fp32 accumulators of the output row per lane
+    if (s.unit == 1 || s.LPN == 0 || s.LPN > 8 || c->K > 256)
+        return fail(c, SDDMM_ERR_UNSUPPORTED,
+                    "the fused SDDMM+SpMM needs K <= 256, a multiple of 4 (fp32) or 8 (bf16, fp16)");
     if (!c->have_rowptr) return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs row-sorted entries");
     rc = plan_fused_items(c);
     if (rc) return rc;
@@ -1441,7 +1443,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
     if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);
-            if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS == 4) {
+            if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS > 1 && LT::UPL * LT::U::ELEMS <= 32) {
                 const int64_t rows_per_wave = WAVE / LT::LPN;
                 const int64_t waves = ((int64_t)c->sM + rows_per_wave - 1) / rows_per_wave;
                 const int64_t rblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;

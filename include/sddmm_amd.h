@@ -216,8 +216,8 @@ int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, cons
  * it (and written like it): the step that consumes an SDDMM result in the applications
  * the reference names.  No counterpart in the reference's code, which stops at P
  * (src/competitors/cpu/cpu_basic.hpp:18-51).  O is M x K fp32 row-major, owned by the
- * context.  Needs fp32 operands with K a multiple of 4 and K <= 256, and row-sorted
- * entries (CSR, or COO with non-decreasing rows); SDDMM_ERR_UNSUPPORTED otherwise.
+ * context.  Needs K <= 256, a multiple of 4 (fp32 operands) or 8 (bf16, fp16), and
+ * row-sorted entries (CSR, or COO with non-decreasing rows); SDDMM_ERR_UNSUPPORTED otherwise.
  * Rows longer than 2048 entries are accumulated with atomic adds, so their last bits
  * may differ from run to run. */
 int sddmm_run_fused(sddmm_ctx *ctx);

@@ -83,11 +83,38 @@ def test_fused_benchmark_shapes_scaled_down(engine_factory, name):
     e.close()
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("K", [8, 32, 64, 136, 256])
+def test_fused_16bit_operands(engine_factory, dtype, K):
+    """bf16 / fp16 A and B (fp32 accumulation, fp32 P and O) against the fp32 oracle on the
+    rounded inputs, short rows (one lane group per row) and rows split into segments."""
+    rng = np.random.default_rng(1300 + K + dtype)
+    M, N = 210, 3000
+    lens = rng.choice([0, 1, 7, 30, 64, 65, 300, 2500], M)
+    rows = [np.sort(rng.choice(N, int(n), replace=False)) for n in lens]
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == capi.BF16:
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        Ar, Br = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K)
+    else:
+        Ab, Bb = capi.to_f16(A).reshape(M, K), capi.to_f16(B).reshape(N, K)
+        Ar, Br = capi.from_f16(Ab).reshape(M, K), capi.from_f16(Bb).reshape(N, K)
+    e = engine_factory()
+    e.set_dense(Ab, Bb, dtype)
+    e.set_csr(M, N, rowptr, col, val)
+    _check(e, rowptr, col, val, Ar, Br, "16-bit K=%d dtype=%d" % (K, dtype))
+    e.close()
+
+
 def test_fused_unsupported_and_state(engine_factory):
     rng = np.random.default_rng(3)
     rowptr = np.array([0, 1, 2], np.int32); col = np.array([1, 0], np.int32); val = np.ones(2, f32)
     e = engine_factory()
-    for K, dt in ((33, capi.F32), (260, capi.F32), (32, capi.BF16)):
+    for K, dt in ((33, capi.F32), (260, capi.F32), (264, capi.BF16)):
         A = rng.uniform(-1, 1, (2, K)).astype(f32)
         if dt == capi.BF16:
             e.set_dense(capi.to_bf16(A).reshape(2, K), capi.to_bf16(A).reshape(2, K), dt)
