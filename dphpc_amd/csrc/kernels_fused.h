@@ -141,14 +141,16 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
 // consecutive rows, group g walks row r0+g.  Lane j of a group reads column index and
 // S value of entry t0+j, so LPN entries of each row are gathered back to back; the
 // P value of entry t0+j ends up in lane j, and the output row needs no reduction
-// across groups.  Longer rows are left to k_fusedmm (they count as empty here); every
-// other row, empty ones included, gets its output row written.
+// across groups.  Longer rows are left to k_fusedmm and the rows of 8-row panels
+// (panel_owner[row] == 2, when the array is given) to the panel kernel (they count as
+// empty here); every other row, empty ones included, gets its output row written.
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                         const int32_t *__restrict__ rowptr,
                                                         const int32_t *__restrict__ col,
                                                         const float *__restrict__ sval, float *__restrict__ P,
-                                                        float *__restrict__ O, int M, int max_len, int64_t nblocks) {
+                                                        float *__restrict__ O, int M, int max_len, int64_t nblocks,
+                                                        const unsigned char *__restrict__ panel_owner) {
     using U = typename L::U;
     using T = typename U::T;
     constexpr int E = U::ELEMS;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
     if (row < M) {
         rs = rowptr[row];
         len = rowptr[row + 1] - rs;
-        mine = len <= max_len;
+        mine = len <= max_len && !(panel_owner && panel_owner[row] == 2);
         if (!mine) len = 0;
     }
     int longest = len;

@@ -210,10 +210,11 @@ constexpr int SCAN_TILE = SCAN_BLOCK * SCAN_ITEMS;  // rows per block
 // owner (may be null): one byte per row, non-zero when the dense-tile path (1: a
 // 16-row strip, 3: a strip of rows gathered by column window) or the row-panel path
 // (2) computes the row; such rows count as empty here
+// (only != 0: just the rows of that owner count as empty)
 __device__ __forceinline__ unsigned int row_item_count(const int32_t *__restrict__ rowptr,
                                                        const unsigned char *__restrict__ owner, int64_t i,
-                                                       int M, int ts, int seg, unsigned int *len_out) {
-    if (i >= M || (owner && owner[i] != 0)) { *len_out = 0; return 0; }
+                                                       int M, int ts, int seg, unsigned int *len_out, int only = 0) {
+    if (i >= M || (owner && (only ? owner[i] == only : owner[i] != 0))) { *len_out = 0; return 0; }
     const unsigned int len = (unsigned int)(rowptr[i + 1] - rowptr[i]);
     *len_out = len;
     return len >= (unsigned int)ts ? (len + seg - 1) / seg : 0u;
@@ -246,13 +247,13 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
                                                                const unsigned char *__restrict__ owner, int M,
                                                                int ts, int seg, unsigned int *__restrict__ block_sums,
-                                                               DevCounters *pc) {
+                                                               DevCounters *pc, int only) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int items = 0;
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        const unsigned int cnt = row_item_count(rowptr, owner, base + q, M, ts, seg, &len);
+        const unsigned int cnt = row_item_count(rowptr, owner, base + q, M, ts, seg, &len, only);
         items += cnt;
         if (len == 0) continue;
         if (cnt == 0) { ++r_short; n_short += len; }
@@ -327,12 +328,12 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_write(const int32_t *__
                                                                const unsigned char *__restrict__ owner, int M,
                                                                int ts, int seg,
                                                                const unsigned int *__restrict__ block_offsets,
-                                                               RowItem *__restrict__ items) {
+                                                               RowItem *__restrict__ items, int only) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int cnt[SCAN_ITEMS], mine = 0;
     for (int q = 0; q < SCAN_ITEMS; ++q) {
         unsigned int len;
-        cnt[q] = row_item_count(rowptr, owner, base + q, M, ts, seg, &len);
+        cnt[q] = row_item_count(rowptr, owner, base + q, M, ts, seg, &len, only);
         mine += cnt[q];
     }
     unsigned int total;

@@ -1286,13 +1286,36 @@ __device__ __forceinline__ void quad_transpose(float (&f)[4], int lane) {
 // with 2 than with 4 at rows of 128-256 bytes, 2-5 % slower at 512 bytes.
 constexpr int panel_mfma_waves(int steps) { return steps <= 4 ? 2 : 4; }
 
-template <int DT, int STEPS>
-__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+// FUSED (fp32, rows of 128 or 256 bytes): the kernel also adds the panel's part of
+//
+//     O[row0+r][:] += sum over the item's columns c of P[row0+r][c] * B[col_c][:]
+//
+// with the same instruction in another role: block b = gathered column b of the group,
+// srcA = the P values of rows 4h.. in that column (lane 4b+i: row 4h+i), srcB = the B
+// unit as it was loaded (lane 4b+j: components 4j.. of unit 4s+j, no layout change), so
+// register i of lane 4b+j of accumulator (h,s,comp) collects O[4h+i][16s+4j+comp] over
+// the columns that block b has seen.  The P values of a pair move from the memory layout
+// to srcA through a tile of LDS (one 16-byte write, four 4-byte reads per lane).  After
+// the last column the 16 blocks are added with lane swaps and row rotations and every
+// lane adds 2*STEPS values to O atomically (O is cleared before the launch; a row may
+// be cut into several items).  Columns past the end of the item enter with srcB = 0,
+// whatever their B rows hold.
+constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;   // rotation by 4 / 8 lanes inside every row of 16
+constexpr int PANEL_TILE_PITCH = 48;                        // floats per row of the P tile: conflict-free 4-byte reads
+
+template <int DT, int STEPS, bool FUSED = false>
+#ifndef SDDMM_FUSED_OCC2
+#define SDDMM_FUSED_OCC2 3
+#define SDDMM_FUSED_OCC4 2
+#endif
+__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, FUSED ? (STEPS == 2 ? SDDMM_FUSED_OCC2 : SDDMM_FUSED_OCC4) : STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const float *__restrict__ sval, float *__restrict__ P,
                                                       const RowItem *__restrict__ items, int64_t n_items,
-                                                      int64_t nblocks) {
+                                                      int64_t nblocks, float *__restrict__ O) {
+    static_assert(!FUSED || (DT == DT_F32 && (STEPS == 2 || STEPS == 4)), "fused panels: fp32 rows of 128 or 256 bytes");
+    __shared__ __attribute__((aligned(16))) float p_tiles[FUSED ? panel_mfma_waves(STEPS) : 1][FUSED ? PANEL_ROWS * PANEL_TILE_PITCH : 4];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     const int64_t w = blk * panel_mfma_waves(STEPS) + wave_in_block();
@@ -1316,7 +1339,10 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
                 : 16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
     constexpr int ROW_UNITS = STEPS * 4;
     // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
-    constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
+#ifndef SDDMM_FUSED_GROUPS
+#define SDDMM_FUSED_GROUPS 4
+#endif
+    constexpr int GROUPS = STEPS >= 8 ? 2 : FUSED ? SDDMM_FUSED_GROUPS : 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     constexpr int A_REGS = BLOCKS ? STEPS / 2 : STEPS;
@@ -1424,6 +1450,34 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
         }
         return acc;
     };
+    // FUSED: accumulator (h, s, comp) of the output rows, see above
+    f32x4_t oacc[2][STEPS][4];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) oacc[h][s][k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    auto fused_accumulate = [&](const Oper &o, float p_lo, float p_hi, int gbase) {
+        const bool live = gbase + lrow < end;                    // this block's column belongs to the item
+#pragma unroll
+        for (int s = 0; s < (FUSED ? STEPS : 0); ++s) {
+            const uint4 b = o.b[s];
+            const unsigned int ux = live ? b.x : 0u, uy = live ? b.y : 0u, uz = live ? b.z : 0u, uw = live ? b.w : 0u;
+            const float bx = __builtin_bit_cast(float, ux), by = __builtin_bit_cast(float, uy);
+            const float bz = __builtin_bit_cast(float, uz), bw = __builtin_bit_cast(float, uw);
+            oacc[0][s][0] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bx, oacc[0][s][0], 0, 0, 0);
+            oacc[1][s][0] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bx, oacc[1][s][0], 0, 0, 0);
+            oacc[0][s][1] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, by, oacc[0][s][1], 0, 0, 0);
+            oacc[1][s][1] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, by, oacc[1][s][1], 0, 0, 0);
+            oacc[0][s][2] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bz, oacc[0][s][2], 0, 0, 0);
+            oacc[1][s][2] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bz, oacc[1][s][2], 0, 0, 0);
+            oacc[0][s][3] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bw, oacc[0][s][3], 0, 0, 0);
+            oacc[1][s][3] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bw, oacc[1][s][3], 0, 0, 0);
+        }
+    };
     // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
     auto compute_store_pair = [&](const Oper &o0, const Oper &o1, int g0) {
         if (g0 >= end) return;                                   // wave-uniform
@@ -1463,16 +1517,34 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
         const float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
         const float d2 = __builtin_bit_cast(float, m.z), d3 = __builtin_bit_cast(float, m.w);
         const int e = g0 + 4 * punit;
+        float p[4] = {0.f, 0.f, 0.f, 0.f};                       // FUSED: the P values, 0 past the end of the item
         if (e + 4 <= end) {
             // four consecutive entries inside the item (so the S window was not clamped)
             F4u out{d0 * o0.s.x, d1 * o0.s.y, d2 * o0.s.z, d3 * o0.s.w};
             *reinterpret_cast<F4u *>(P + out_row + e) = out;
+            p[0] = out.x; p[1] = out.y; p[2] = out.z; p[3] = out.w;
         } else {
             // the item ends inside these four: entry by entry, S values fetched again
             const float d[4] = {d0, d1, d2, d3};
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (e + i < end) P[out_row + e + i] = d[i] * sval[out_row + e + i];
+                if (e + i < end) {
+                    p[i] = d[i] * sval[out_row + e + i];
+                    P[out_row + e + i] = p[i];
+                }
+        }
+        if constexpr (FUSED) {
+            float *tile = p_tiles[wave_in_block()];
+            const f32x4_t pv = {p[0], p[1], p[2], p[3]};
+            *reinterpret_cast<f32x4_t *>(tile + prow * PANEL_TILE_PITCH + 4 * punit) = pv;
+            wave_lds_order();
+            // lane 4b+i: row 4h+i, column b of the first / second group
+            const float *src = tile + (lane & 3) * PANEL_TILE_PITCH + lrow;
+            const float p0_lo = src[0], p0_hi = src[4 * PANEL_TILE_PITCH];
+            const float p1_lo = src[16], p1_hi = src[4 * PANEL_TILE_PITCH + 16];
+            wave_lds_order();
+            fused_accumulate(o0, p0_lo, p0_hi, g0);
+            fused_accumulate(o1, p1_lo, p1_hi, g0 + 16);
         }
     };
 
@@ -1500,6 +1572,34 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, STEPS == 8 ? 4 : 1)
             o[u + 1] = load_oper(cc_nxt, u + 1, base + CHUNK + 16 * u + 16);
         }
         cc_nxt = cc_nn;
+    }
+    if constexpr (FUSED) {
+        // Register i of lane 4b+j of accumulator (h,s,comp) is O[4h+i][16s+4j+comp] over block b's
+        // columns.  The swaps add the four rows of 16 lanes while dealing the registers out: row r
+        // of the wave keeps register {0,2,1,3}[r]; the rotations add the four blocks of a row.  All
+        // four blocks then hold the same 16 sums; block cg adds the ones of component cg to O.
+        const int r16 = lane >> 4, cg = (lane >> 2) & 3;
+        const int orow = row0 + ((r16 & 1) << 1 | (r16 >> 1));
+        constexpr int K = STEPS * 16;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                float w4[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const f32x4_t v = oacc[h][s][k];
+                    const float t0 = swap32_add(v[0], v[1]);
+                    const float t1 = swap32_add(v[2], v[3]);
+                    float x = swap16_add(t0, t1);
+                    x += dpp_f32<DPP_ROW_ROR4>(x);
+                    x += dpp_f32<DPP_ROW_ROR8>(x);
+                    w4[k] = x;
+                }
+                const float mine = cg == 0 ? w4[0] : cg == 1 ? w4[1] : cg == 2 ? w4[2] : w4[3];
+                atomicAdd(O + (int64_t)(orow + 4 * h) * K + 16 * s + 4 * (lane & 3) + cg, mine);
+            }
+        }
     }
 }
 

@@ -110,6 +110,7 @@ struct sddmm_ctx {
     RowItem *d_fused_items = nullptr;
     int64_t n_fused_items = 0, fused_items_cap = 0;
     bool fused_items_valid = false;
+    bool fused_items_panels = false; // the fused items leave out the rows that the panel kernel owns
     float *dO = nullptr;
     size_t o_cap = 0;
     bool have_fused = false;
@@ -484,7 +485,7 @@ int classify_rows_count(sddmm_ctx *c, bool again = false) {
     if (nb > 0) {
         const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr, owner,
-                           c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc);
+                           c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc, 0);
         SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
         LAUNCH_CHECK(c);
@@ -506,7 +507,7 @@ int classify_rows_items(sddmm_ctx *c) {
     if (c->n_items > 0) {
         SDDMM_LAUNCH(c, k_classify_write, nb, SCAN_BLOCK, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts, c->seg,
-                           c->d_block_sums, c->d_items);
+                           c->d_block_sums, c->d_items, 0);
         LAUNCH_CHECK(c);
     }
     return SDDMM_OK;
@@ -786,7 +787,16 @@ void launch_panel_mfma_t(sddmm_ctx *c) {
     const int64_t nblocks = (c->n_panel_items + PW - 1) / PW;
     SDDMM_LAUNCH(c, (k_panel_mfma<DT, STEPS>), xcd_grid(nblocks), PW * WAVE,
                        (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
-                       c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks);
+                       c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks, (float *)nullptr);
+}
+// the panels of the fused SDDMM+SpMM: P and the panels' part of O
+template <int STEPS>
+void launch_panel_fused_t(sddmm_ctx *c) {
+    constexpr int PW = panel_mfma_waves(STEPS);
+    const int64_t nblocks = (c->n_panel_items + PW - 1) / PW;
+    SDDMM_LAUNCH(c, (k_panel_mfma<DT_F32, STEPS, true>), xcd_grid(nblocks), PW * WAVE,
+                       (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
+                       c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks, c->dO);
 }
 template <int DT>
 void launch_panel_mfma_steps(sddmm_ctx *c) {
@@ -927,6 +937,7 @@ int do_plan(sddmm_ctx *c, int strategy) {
     // the plan state is rewritten in place: a plan that fails half way must not leave the
     // previous one looking valid (its items exclude rows that tiles and panels owned)
     c->planned = false;
+    c->fused_items_valid = false;    // they leave out the rows of this plan's panels
     int resolved = strategy;
     const bool csr_ok = c->have_rowptr;
     // without a row pointer (unsorted COO) only the flat kernels apply
@@ -1381,8 +1392,8 @@ int sddmm_run(sddmm_ctx *c) {
 }
 
 // items of the fused kernel: the rows of more than FUSED_ROW_MAX entries, cut into segments of SDDMM_SEG entries
-static int plan_fused_items(sddmm_ctx *c) {
-    if (c->fused_items_valid) return SDDMM_OK;
+static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
+    if (c->fused_items_valid && c->fused_items_panels == (panel_owner != nullptr)) return SDDMM_OK;
     const int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     const int arc = ensure_arena(c);
@@ -1394,7 +1405,7 @@ static int plan_fused_items(sddmm_ctx *c) {
     c->n_fused_items = 0;
     if (nb > 0) {
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr,
-                           (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc);
+                           panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc, 2);
         SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
         LAUNCH_CHECK(c);
@@ -1409,11 +1420,12 @@ static int plan_fused_items(sddmm_ctx *c) {
         }
         if (c->n_fused_items > 0) {
             SDDMM_LAUNCH(c, k_classify_write, nb, SCAN_BLOCK, c->d_rowptr,
-                               (const unsigned char *)nullptr, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_fused_items);
+                               panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_fused_items, 2);
             LAUNCH_CHECK(c);
         }
     }
     c->fused_items_valid = true;
+    c->fused_items_panels = panel_owner != nullptr;
     return SDDMM_OK;
 }
 
@@ -1428,7 +1440,18 @@ int sddmm_run_fused(sddmm_ctx *c) {
         return fail(c, SDDMM_ERR_UNSUPPORTED,
                     "the fused SDDMM+SpMM needs K <= 256, a multiple of 4 (fp32) or 8 (bf16, fp16)");
     if (!c->have_rowptr) return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs row-sorted entries");
-    rc = plan_fused_items(c);
+    // fp32 rows of 128 or 256 bytes: the 8-row panels of the current plan (AUTO if there is none
+    // yet) take the matrix-core kernel, which shares every gathered B row between 8 rows and both
+    // products; the other rows take the gather kernels
+    bool panels = c->dtype == SDDMM_F32 && (c->K == 32 || c->K == 64) && env_int("SDDMM_FUSED_PANELS", 1) != 0;
+    if (panels && !c->planned) {
+        rc = sddmm_plan(c, c->requested);
+        if (rc) return rc;
+    }
+    panels = panels && c->planned && c->panel_mfma && c->n_panel_items > 0 && c->owner_active &&
+             (c->strategy == SDDMM_AUTO || c->strategy == SDDMM_LDS_TILED || c->strategy == SDDMM_MFMA_TILE);
+    const unsigned char *panel_owner = panels ? (const unsigned char *)c->d_owner : nullptr;
+    rc = plan_fused_items(c, panel_owner);
     if (rc) return rc;
     const size_t o_bytes = (size_t)c->M * (size_t)c->K * sizeof(float);
     if (o_bytes > c->o_cap) {
@@ -1443,13 +1466,16 @@ int sddmm_run_fused(sddmm_ctx *c) {
     if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);
+            // (when the panels own every row that has entries, O is complete after the memset and the panel kernel)
+            const bool others = !panels || c->n_tiles > 0 || c->rows_short > 0 || c->n_items > 0;
+            if (!others) return;
             if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS > 1 && LT::UPL * LT::U::ELEMS <= 32) {
                 const int64_t rows_per_wave = WAVE / LT::LPN;
                 const int64_t waves = ((int64_t)c->sM + rows_per_wave - 1) / rows_per_wave;
                 const int64_t rblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
                 SDDMM_LAUNCH(c, (k_fusedmm_rows<LT>), xcd_grid(rblocks), BLOCK,
                                    (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
-                                   c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks);
+                                   c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks, panel_owner);
                 ++launches;
                 if (c->n_fused_items > 0) {
                     const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
@@ -1461,6 +1487,11 @@ int sddmm_run_fused(sddmm_ctx *c) {
                 }
             }
         });
+        if (panels) {
+            if (c->K == 32) launch_panel_fused_t<2>(c);
+            else launch_panel_fused_t<4>(c);
+            ++launches;
+        }
         LAUNCH_CHECK(c);
     }
     HIP_TRY(c, hipEventRecord(c->ev1, c->stream));

@@ -174,3 +174,95 @@ def test_fused_non_finite_rows_of_b_stay_in_their_own_entries(engine_factory):
     clean = ~bad_row
     np.testing.assert_allclose(got_o[clean], ref_o[clean], rtol=1e-4, atol=1e-5)
     e.close()
+
+
+def _panel_pattern(rng, N, panel_lens, loose_lens):
+    """8-row panels (one column list per panel) with loose rows in between, in groups of 8 so
+    that the panels stay 8-aligned."""
+    rows = []
+    for i, n in enumerate(panel_lens):
+        cols = np.sort(rng.choice(N, int(n), replace=False))
+        rows += [cols] * 8
+        if i < len(loose_lens):
+            rows += [np.sort(rng.choice(N, int(m), replace=False)) for m in loose_lens[i]]
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    return len(rows), rowptr, col
+
+
+@pytest.mark.parametrize("K", [32, 64])
+@pytest.mark.parametrize("strategy", [capi.AUTO, capi.LDS_TILED])
+def test_fused_row_panels_on_the_matrix_cores(engine_factory, monkeypatch, K, strategy):
+    """fp32 rows of 128 / 256 bytes: the 8-row panels of the plan take the panel kernel (P and O
+    from one pass over the gathered B rows), the other rows the gather kernels.  Panel lengths
+    around the group sizes (16, 32, 64 columns) and items that cut a panel's list."""
+    monkeypatch.setenv("SDDMM_PANEL_SEG", "128")
+    rng = np.random.default_rng(4100 + K + strategy)
+    N = 1500
+    panel_lens = [4, 5, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300, 700]
+    loose = [[0, 3, 70, 1, 0, 200, 9, 64]] * 5 + [[12] * 8] * 3
+    M, rowptr, col = _panel_pattern(rng, N, panel_lens, loose)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    e.plan(strategy)
+    out = _check(e, rowptr, col, val, A, B, "panels K=%d strategy=%d" % (K, strategy))
+    assert e.stats().kernels_launched == 3               # short rows, long rows, panels
+    monkeypatch.setenv("SDDMM_FUSED_PANELS", "0")
+    plain = _check(e, rowptr, col, val, A, B, "panels off")
+    assert e.stats().kernels_launched == 2
+    np.testing.assert_allclose(out, plain, rtol=1e-4, atol=1e-5)
+    monkeypatch.delenv("SDDMM_FUSED_PANELS")
+    # the SDDMM alone still works on the same plan, and a new plan without panels drops them
+    e.run()
+    ok, _, _ = O.check_values(e.values(), O.sddmm_csr(rowptr, col, val, A, B), mag=O.sddmm_csr_f64(rowptr, col, val, A, B)[1])
+    assert ok
+    e.plan(capi.FLAT)
+    _check(e, rowptr, col, val, A, B, "after a plan without panels")
+    assert e.stats().kernels_launched == 2
+    e.close()
+
+
+def test_fused_row_panels_keep_non_finite_b_rows_in_their_own_entries(engine_factory, monkeypatch):
+    """A panel's list is cut into items of 128 columns and ends in the middle of a group of 16:
+    the groups past an item's end load the B row of a clamped position, and the first column of
+    the next item holds an infinity.  Neither may reach the output rows through 0 * inf."""
+    monkeypatch.setenv("SDDMM_PANEL_SEG", "128")
+    rng = np.random.default_rng(88)
+    N, K = 900, 32
+    M, rowptr, col = _panel_pattern(rng, N - 2, [150, 37, 200], [])
+    rowptr = rowptr.copy(); col = col.copy()
+    lens = np.diff(rowptr)
+    # panel 1 (rows 8..15, 37 columns): its last column is B row N-1 (NaN); panel 2: column 128 of the list is B row N-2 (inf)
+    for r in range(8, 16):
+        col[rowptr[r] + 36] = N - 1
+    for r in range(16, 24):
+        seg = col[rowptr[r]:rowptr[r + 1]]
+        seg[128:] = np.sort(np.concatenate([[N - 2], seg[129:]]))
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    B[N - 2, 5] = np.inf
+    B[N - 1, 20] = np.nan
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    e.plan(capi.AUTO)
+    got_o = e.run_fused()
+    assert e.stats().kernels_launched == 1               # every row belongs to a panel
+    got_p = e.values()
+    with np.errstate(all="ignore"):
+        ref_p, ref_o = O.fusedmm_csr(rowptr, col, val, A, B)
+    bad_entry = (col == N - 2) | (col == N - 1)
+    assert np.array_equal(~np.isfinite(got_p), bad_entry)
+    bad_row = np.zeros(M, bool)
+    bad_row[np.repeat(np.arange(M), lens)[bad_entry]] = True
+    assert bad_row[8:24].all() and not bad_row[:8].any()
+    assert np.array_equal(~np.isfinite(got_o).all(axis=1), bad_row)
+    np.testing.assert_allclose(got_o[:8], ref_o[:8], rtol=1e-4, atol=1e-5)
+    assert np.array_equal(np.isfinite(got_o), np.isfinite(ref_o))
+    e.close()
