@@ -80,6 +80,19 @@ def test_structured_random(engine_factory, seed):
         if st.strategy_used in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED):
             owned = st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long
             assert owned == len(col), (seed, capi.STRATEGY_NAMES[strategy], st.as_dict())
+    # SDDMM followed by SpMM on the same mixture: the panels of the plan take their own kernel,
+    # rows that tiles own in the SDDMM take the gather kernels
+    if K % 4 == 0:
+        ref_p, ref_o = O.fusedmm_csr(rowptr, col, val, A, B)
+        _, mag_o = O.fusedmm_csr_f64(rowptr, col, val, A, B)
+        for strategy in (capi.AUTO, capi.LDS_TILED):
+            e.set_csr(M, N, rowptr, col, val)
+            e.plan(strategy)
+            got_o = e.run_fused()
+            ok, worst, i = O.check_values(e.values(), ref, mag=mag)
+            assert ok, (seed, "fused P", capi.STRATEGY_NAMES[strategy], i, worst)
+            ok, worst, i = O.check_values(got_o[:M].ravel(), ref_o.ravel(), mag=mag_o.ravel())
+            assert ok, (seed, "fused O", capi.STRATEGY_NAMES[strategy], i, worst)
     # bf16 on the same structure
     Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
     if K % 8 == 0:
