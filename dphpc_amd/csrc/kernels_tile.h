@@ -285,7 +285,22 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
             const int words = (span + 31) >> 5;
             for (int w = lane; w < words; w += WAVE) bm[w] = 0u;
             wave_lds_order();
-            const int64_t ch = strip_scan<1>(col, e0, e1, budget, lo, span, bm, &descents);
+            // Rows 0 and 8 first: their tile columns alone often exceed what the strip may have
+            // (two 8-row blocks with different column lists), and the other 14 rows are then
+            // never read.  The bits stay: the scan of the whole strip sets them again.
+            int64_t ch = 0;
+            if (entries > 4 * FIRST) {
+                int64_t unused;
+                const int a0 = e0, a1 = __builtin_amdgcn_readlane(lane_rp, 1);
+                const int b0 = __builtin_amdgcn_readlane(lane_rp, 8), b1 = __builtin_amdgcn_readlane(lane_rp, 9);
+                if (a1 > a0) (void)strip_scan<1>(col, a0, a1, INT64_MAX, lo, span, bm, &unused);
+                if (b1 > b0) (void)strip_scan<1>(col, b0, b1, INT64_MAX, lo, span, bm, &unused);
+                wave_lds_order();
+                int t = 0;
+                for (int w = lane; w < words; w += WAVE) t += __builtin_popcount(bm[w]);
+                if (wave_sum_i32(t) > max_tiles) ch = -1;
+            }
+            if (ch >= 0) ch = strip_scan<1>(col, e0, e1, budget, lo, span, bm, &descents);
             wave_lds_order();
             if (ch >= 0 && descents == allowed) {
                 int t = 0;
