@@ -285,6 +285,33 @@ def test_context_reuse_and_update_values(engine_factory):
     e.close()
 
 
+def test_one_context_across_patterns_of_different_sizes(engine_factory):
+    """One context, as the harness keeps one competitor object: patterns with more and fewer
+    rows, entries, tiles and panels in turn.  The plan's work arrays are sized for the largest
+    pattern seen; a smaller one after a larger one must not see what the larger one left."""
+    e = engine_factory()
+    order = ["mixed_density", "small_uniform", "fem_banded", "dense_tiles", "small_uniform", "mixed_density",
+             "power_law", "fem_banded"]
+    for name in order:
+        w = W.make(name, "small", K=32)
+        e.set_dense(w.A, w.B)
+        e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+        for strategy in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED):
+            e.plan(strategy)
+            e.run()
+            st = e.stats()
+            assert_parity(e.values(), w.rowptr, w.col, w.sval, w.A, w.B, what="%s after others" % name)
+            if st.strategy_used in (capi.AUTO, capi.MFMA_TILE, capi.LDS_TILED):
+                assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == w.nnz
+        e.plan(capi.AUTO)
+        got_o = e.run_fused()
+        ref_p, ref_o = O.fusedmm_csr(w.rowptr, w.col, w.sval, w.A, w.B)
+        _, mag_o = O.fusedmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+        ok, worst, i = O.check_values(got_o[:w.M].ravel(), ref_o.ravel(), mag=mag_o.ravel())
+        assert ok, (name, i, worst)
+    e.close()
+
+
 @pytest.mark.parametrize("name", ["fem_banded", "mixed_density", "similar_rows"])
 def test_non_finite_operands_stay_in_their_own_entries(engine_factory, name):
     """A NaN in one B row and an infinity in one A row: exactly the entries that involve
