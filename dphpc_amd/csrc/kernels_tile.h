@@ -1323,13 +1323,13 @@ template <int DT, int STEPS, bool FUSED = false>
 #define SDDMM_FUSED_OCC2 3
 #define SDDMM_FUSED_OCC4 2
 #endif
-__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, FUSED ? (STEPS == 2 ? SDDMM_FUSED_OCC2 : SDDMM_FUSED_OCC4) : STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, FUSED ? (STEPS == 2 ? SDDMM_FUSED_OCC2 : STEPS == 4 ? SDDMM_FUSED_OCC4 : 1) : STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const float *__restrict__ sval, float *__restrict__ P,
                                                       const RowItem *__restrict__ items, int64_t n_items,
                                                       int64_t nblocks, float *__restrict__ O) {
-    static_assert(!FUSED || (DT == DT_F32 && (STEPS == 2 || STEPS == 4)), "fused panels: fp32 rows of 128 or 256 bytes");
+    static_assert(!FUSED || (DT == DT_F32 && (STEPS == 2 || STEPS == 4 || STEPS == 8)), "fused panels: fp32 rows of 128 to 512 bytes");
     __shared__ __attribute__((aligned(16))) float p_tiles[FUSED ? panel_mfma_waves(STEPS) : 1][FUSED ? PANEL_ROWS * PANEL_TILE_PITCH : 4];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;

@@ -1443,7 +1443,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
     // fp32 rows of 128 or 256 bytes: the 8-row panels of the current plan (AUTO if there is none
     // yet) take the matrix-core kernel, which shares every gathered B row between 8 rows and both
     // products; the other rows take the gather kernels
-    bool panels = c->dtype == SDDMM_F32 && (c->K == 32 || c->K == 64) && env_int("SDDMM_FUSED_PANELS", 1) != 0;
+    bool panels = c->dtype == SDDMM_F32 && (c->K == 32 || c->K == 64 || c->K == 128) && env_int("SDDMM_FUSED_PANELS", 1) != 0;
     if (panels && !c->planned) {
         rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
@@ -1489,7 +1489,8 @@ int sddmm_run_fused(sddmm_ctx *c) {
         });
         if (panels) {
             if (c->K == 32) launch_panel_fused_t<2>(c);
-            else launch_panel_fused_t<4>(c);
+            else if (c->K == 64) launch_panel_fused_t<4>(c);
+            else launch_panel_fused_t<8>(c);
             ++launches;
         }
         LAUNCH_CHECK(c);

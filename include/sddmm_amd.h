@@ -220,7 +220,7 @@ int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, cons
  * row-sorted entries (CSR, or COO with non-decreasing rows); SDDMM_ERR_UNSUPPORTED otherwise.
  * Rows longer than 2048 entries are accumulated with atomic adds, so their last bits
  * may differ from run to run.
- * fp32 operands with K = 32 or 64: the rows that the current plan (SDDMM_AUTO is planned
+ * fp32 operands with K = 32, 64 or 128: the rows that the current plan (SDDMM_AUTO is planned
  * if there is none) runs as 8-row panels take a matrix-core kernel that shares every
  * gathered B row between the 8 rows and between both products; panels whose column list
  * is cut into several work items (more than 512 columns) are accumulated with atomic adds
