@@ -211,6 +211,31 @@ def time_strategy(e, w, capi, name, steps, warmup, flusher, checker, cold_reps=6
         raise
 
 
+def fused_leg(e, w, capi, reps, check):
+    """O = P * B after the SDDMM, in the same pass (sddmm_run_fused): device time per call between
+    the library's own events (the memset of O included), 4*nnz*K flops."""
+    e.plan(capi.AUTO)
+    times = []
+    for _ in range(reps):
+        e.run_fused(fetch=False)
+        times.append(e.stats().run_ms)
+    launches = e.stats().kernels_launched
+    t = float(np.median(times))
+    res = {"ms_p50": t, "ms_min": float(min(times)), "gflops": 4.0 * w.nnz * w.K / (t * 1e-3) / 1e9,
+           "kernels_launched": launches, "validated": None}
+    if check:
+        from oracle import oracle as O
+        got = e.run_fused()
+        ref_p, ref_o = O.fusedmm_csr(w.rowptr, w.col, w.sval, w.A, w.B)
+        _, mag_o = O.fusedmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+        ok, worst, i = O.check_values_fast(got[:w.M].ravel(), ref_o.ravel(), mag=mag_o.ravel(), rtol=rtol_for(w, "AUTO"))
+        if not ok:
+            log("VALIDATION FAILED (fused): element %d got %r (%.2f x tolerance)" % (i, got[:w.M].ravel()[i], worst))
+            sys.exit(1)
+        res["validated"] = {"elements": int(w.M * w.K), "worst_over_tol": round(worst, 4)}
+    return res
+
+
 def fractions(w, us, cold_us):
     """Compulsory bytes over launch time against the HBM peak (and the dense-tile
     shape's flops against the bf16 MFMA peak)."""
@@ -281,6 +306,8 @@ def main():
     ap.add_argument("--per-config", default=None, choices=["full", "small", "none"],
                     help="size of the per_config sweep (default: full with --size full, none otherwise)")
     ap.add_argument("--no-per-config", action="store_true", help="headline only (e.g. under a profiler)")
+    ap.add_argument("--fused", action="store_true",
+                    help="also time SDDMM followed by SpMM over the same pattern (sddmm_run_fused) and add it as `fused`")
     args = ap.parse_args()
 
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -401,6 +428,8 @@ def main():
                     "nnz_mfma": st.nnz_mfma},
         "validated": validated,
     }
+    if args.fused:
+        out["fused"] = fused_leg(e, w, capi, max(args.steps, 20), not args.no_check)
     e.close()
     if not args.no_cpu:
         base, allc = cpu_baseline(w)

@@ -239,9 +239,12 @@ class Engine:
         self._chk(self.L.sddmm_time_region(self.h, reps, int(include_plan), C.byref(total)))
         return float(total.value)
 
-    def run_fused(self):
-        """SDDMM followed by SpMM over the same pattern; returns O (M x K, fp32)."""
+    def run_fused(self, fetch=True):
+        """SDDMM followed by SpMM over the same pattern; returns O (M x K, fp32), or nothing
+        with fetch=False (stats().run_ms then holds the device time of the launch)."""
         self._chk(self.L.sddmm_run_fused(self.h))
+        if not fetch:
+            return None
         O = np.empty(self._dense_shape, np.float32)
         self._chk(self.L.sddmm_get_fused(self.h, _ptr(O)))
         return O

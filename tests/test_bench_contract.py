@@ -28,7 +28,7 @@ def test_traffic_table_names_existing_profiles():
 @pytest.mark.gpu
 def test_json_line_on_a_small_run():
     p = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--size", "small", "--steps", "5", "--warmup", "2",
-                        "--per-config", "small"],
+                        "--per-config", "small", "--fused"],
                        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=280)
     assert p.returncode == 0, p.stderr
     lines = [l for l in p.stdout.splitlines() if l.strip()]
@@ -49,6 +49,9 @@ def test_json_line_on_a_small_run():
     c = d["cpu_baseline"]
     assert c["kind"] in ("reference", "port") and c["cores"] == 1 and c["value"] > 0 and c["sample"]
     assert d["validated"]["entries"] == d["config"]["nnz"]
+    f = d["fused"]
+    assert f["ms_p50"] >= f["ms_min"] > 0 and f["kernels_launched"] >= 1
+    assert f["validated"]["elements"] == d["config"]["M"] * d["config"]["K"] and f["validated"]["worst_over_tol"] <= 1.0
     # the sweep over the five shapes: AUTO next to every fixed strategy, all validated
     pc = d["per_config"]
     assert [(x["workload"], x["K"]) for x in pc] == [
