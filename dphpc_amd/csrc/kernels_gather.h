@@ -345,6 +345,39 @@ __device__ __forceinline__ void short_rows_body(const void *__restrict__ A, cons
     }
 }
 
+// One wavefront, entries [64 chunk, 64 chunk + 64) of the plan's entry list of the short rows
+// ({position, row} per entry, k_short_list_write): the flat kernel's body on a subset of the
+// entries.  Three dependent round trips (list, index and S value, gathers) and full lanes
+// whatever the row lengths; short_rows_body pays two round trips and a dozen lane exchanges
+// before its first index load and one more round trip per chunk.
+template <class L>
+__device__ __forceinline__ void entry_list_body(const void *__restrict__ A, const void *__restrict__ B, int KU,
+                                                const int2 *__restrict__ list, int64_t n_list,
+                                                const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                float *__restrict__ P, int64_t chunk, int lane) {
+    using U = typename L::U;
+    using T = typename U::T;
+    const int64_t base = chunk * WAVE;
+    if (base >= n_list) return;
+    const int64_t left = n_list - base;
+    const int count = left < WAVE ? (int)left : WAVE;
+    const bool valid = lane < count;
+    const int2 pr = list[base + (valid ? lane : count - 1)];   // lanes past the end repeat the last entry
+    const int c = ld_stream(col + pr.x);
+    const float s = ld_stream(sval + pr.x);
+    float res;
+    if constexpr (L::LONG) {
+        res = chunk_long<U>((const T *)A, (const T *)B, KU, c, pr.y, count, lane);
+    } else {
+        using C = Chunk<U, L::LPN, L::UPL, L::FULLK, true, L::WIDE>;
+        using O = typename C::O;
+        const O rb = (O)KU * (O)sizeof(T);
+        typename C::Areg none;
+        res = C::run(A, B, KU, none, (O)c * rb, (O)pr.y * rb, count, lane, []() {});
+    }
+    if (valid) st_stream(P + pr.x, res * s);
+}
+
 // ---------------------------------------------------------------------------
 // ROW_WAVE: one wavefront per work item.  With items == nullptr item w is the
 // whole row w.
@@ -403,7 +436,8 @@ __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, cons
                                                 const float *__restrict__ sval, float *__restrict__ P, int M,
                                                 int ts, int rpw, int64_t short_blocks,
                                                 const RowItem *__restrict__ items, int64_t n_items,
-                                                int64_t nblocks) {
+                                                int64_t nblocks, const int2 *__restrict__ short_list,
+                                                int64_t n_short_list) {
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     // interleave: the item blocks of a long-row-heavy matrix start early instead
@@ -421,6 +455,11 @@ __global__ __launch_bounds__(BLOCK) void k_auto(const void *__restrict__ A, cons
         row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
     } else {
         const int64_t sb = blk - items_before;
+        if (short_list) {
+            entry_list_body<L>(A, B, KU, short_list, n_short_list, col, sval, P, sb * WAVES_PER_BLOCK + wave_in_block(),
+                               lane_id());
+            return;
+        }
         const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
         if (r0 >= M) return;
         short_rows_body<L>(A, B, KU, rowptr, owner, col, sval, P, M, ts, r0, rpw, lane_id());

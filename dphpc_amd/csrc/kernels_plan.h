@@ -35,7 +35,7 @@ struct DevCounters {
     unsigned int bad_pattern, coo_unsorted, pad0, pad1;
     unsigned long long n_items, tiles_scanned, panel_items;          // scan totals, one writer each
     unsigned long long n_candidates;                                 // rows offered to the gathered strips
-    unsigned long long utiles_scanned, pad3;                         // scan total of the union strips
+    unsigned long long utiles_scanned, short_scanned;                // scan totals: union strips, entries of the short rows
     unsigned int max_len[SPREAD];
     unsigned long long k[K_KINDS][SPREAD];
 };
@@ -94,9 +94,9 @@ __global__ __launch_bounds__(256) void k_plan_reset(unsigned char *__restrict__ 
             for (int sl = threadIdx.x; sl < SPREAD; sl += blockDim.x) pc->k[k][sl] = 0ull;
         if (threadIdx.x == 0) {
             pc->n_items = 0ull;
+            pc->short_scanned = 0ull;
             if (!rows_only) {
                 pc->tiles_scanned = 0ull; pc->panel_items = 0ull; pc->n_candidates = 0ull; pc->utiles_scanned = 0ull;
-                pc->pad3 = 0ull;
             }
         }
     }
@@ -247,7 +247,8 @@ __device__ __forceinline__ unsigned int block_exclusive_scan(unsigned int v, uns
 __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__restrict__ rowptr,
                                                                const unsigned char *__restrict__ owner, int M,
                                                                int ts, int seg, unsigned int *__restrict__ block_sums,
-                                                               DevCounters *pc, int only) {
+                                                               DevCounters *pc, int only,
+                                                               unsigned int *__restrict__ short_sums) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     unsigned int items = 0;
     unsigned long long r_short = 0, r_med = 0, r_long = 0, n_short = 0, n_med = 0, n_long = 0;
@@ -279,6 +280,8 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_classify_count(const int32_t *__
     }
     __syncthreads();
     if (threadIdx.x < 6) spread_add(pc, K_ROWS_SHORT + (int)threadIdx.x, sh[threadIdx.x]);
+    // entries of this block's short rows, for the entry list (k_short_list_write)
+    if (short_sums && threadIdx.x == 0) short_sums[blockIdx.x] = (unsigned int)sh[3];
 }
 
 // pass 2: exclusive scan of the block sums in place (one workgroup), total -> *total_out
@@ -321,6 +324,36 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_small(const unsigned int *_
         carry += total;
     }
     if (threadIdx.x == 0) *total_out = carry;
+}
+
+// The entry list of the short rows: {position, row} of every stored entry of the rows that
+// have fewer than ts entries and no owner, in storage order.  The kernels take it 64 entries
+// per wavefront, whatever the lengths of the rows (block_offsets: exclusive scan of the
+// short_sums of k_classify_count).
+__global__ __launch_bounds__(SCAN_BLOCK) void k_short_list_write(const int32_t *__restrict__ rowptr,
+                                                                 const unsigned char *__restrict__ owner, int M,
+                                                                 int ts, const unsigned int *__restrict__ block_offsets,
+                                                                 int2 *__restrict__ list) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    unsigned int len[SCAN_ITEMS], mine = 0;
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        const int64_t i = base + q;
+        unsigned int l = 0;
+        if (i < M && !(owner && owner[i] != 0)) {
+            l = (unsigned int)(rowptr[i + 1] - rowptr[i]);
+            if (l >= (unsigned int)ts) l = 0;
+        }
+        len[q] = l;
+        mine += l;
+    }
+    unsigned int total;
+    unsigned int at = block_offsets[blockIdx.x] + block_exclusive_scan(mine, &total);
+    for (int q = 0; q < SCAN_ITEMS; ++q) {
+        if (len[q] == 0) continue;
+        const int32_t row = (int32_t)(base + q);
+        const int32_t rs = rowptr[row];
+        for (unsigned int e = 0; e < len[q]; ++e) list[at++] = make_int2(rs + (int32_t)e, row);
+    }
 }
 
 // pass 3: write the items

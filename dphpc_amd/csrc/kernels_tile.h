@@ -1160,7 +1160,8 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
                                                       const int32_t *__restrict__ tile_cols,
                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                       const TileWindow *__restrict__ win, int64_t n_win, int64_t nnz,
-                                                      int64_t tile_blocks, int64_t nblocks) {
+                                                      int64_t tile_blocks, int64_t nblocks,
+                                                      const int2 *__restrict__ short_list, int64_t n_short_list) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
@@ -1184,6 +1185,11 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
         row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
     } else {
         const int64_t sb = rb - items_before;
+        if (short_list) {
+            entry_list_body<L>(A, B, KU, short_list, n_short_list, col, sval, P, sb * WAVES_PER_BLOCK + wave_in_block(),
+                               lane_id());
+            return;
+        }
         const int64_t r0 = (sb * WAVES_PER_BLOCK + wave_in_block()) * rpw;
         if (r0 >= M) return;
         short_rows_body<L>(A, B, KU, rowptr, owner, col, sval, P, M, ts, r0, rpw, lane_id());

@@ -102,6 +102,10 @@ struct sddmm_ctx {
     // row-panel path
     unsigned int *d_panel_counts = nullptr, *d_panel_off = nullptr;
     int64_t panels_cap = 0;
+    int2 *d_short_list = nullptr;    // {position, row} of the entries of the short rows nobody owns
+    int64_t n_short_list = 0, short_list_cap = 0;
+    bool use_short_list = false;
+    unsigned int *d_short_sums = nullptr;   // arena view: entries of short rows per block of the row scan
     RowItem *d_panel_items = nullptr;
     int64_t n_panel_items = 0, panel_items_cap = 0, n_panels = 0, nnz_panels = 0;
     bool panel_mfma = false;         // panels run on k_panel_mfma (else on k_panel)
@@ -188,7 +192,7 @@ void release_arena(sddmm_ctx *c) {
     c->d_panel_counts = c->d_panel_off = c->d_vstrip_ntiles = c->d_vstrip_off = nullptr;
     c->d_cand_keys = c->d_sorted_keys = nullptr;
     c->d_vrows = nullptr;
-    c->d_block_sums = nullptr;
+    c->d_block_sums = c->d_short_sums = nullptr;
     c->owner_cap = c->strips_cap = c->ustrips_cap = c->panels_cap = c->cand_cap = c->vstrips_cap = 0;
     c->block_sums_cap = 0;
 }
@@ -211,7 +215,7 @@ int ensure_arena(sddmm_ctx *c) {
     const size_t o_vrows = take((size_t)n_strips * 16 * 4);
     const size_t o_panel_n = take((size_t)n_panels * 4), o_panel_o = take((size_t)n_panels * 4);
     const size_t o_keys = take((size_t)(M + 1) * 8), o_sorted = take((size_t)(M + 1) * 8);
-    const size_t o_sums = take((size_t)n_sums * 4);
+    const size_t o_sums = take((size_t)n_sums * 4), o_short_sums = take((size_t)n_sums * 4);
     ALLOC_TRY(c, c->d_arena, at);
     char *b = c->d_arena;
     c->d_owner = (unsigned char *)(b + o_owner);
@@ -222,6 +226,7 @@ int ensure_arena(sddmm_ctx *c) {
     c->d_panel_counts = (unsigned int *)(b + o_panel_n); c->d_panel_off = (unsigned int *)(b + o_panel_o);
     c->d_cand_keys = (unsigned long long *)(b + o_keys); c->d_sorted_keys = (unsigned long long *)(b + o_sorted);
     c->d_block_sums = (unsigned int *)(b + o_sums);
+    c->d_short_sums = (unsigned int *)(b + o_short_sums);
     c->owner_cap = M + 64;
     c->strips_cap = c->ustrips_cap = c->vstrips_cap = n_strips;
     c->panels_cap = n_panels;
@@ -264,6 +269,9 @@ void release_sparse(sddmm_ctx *c) {
     c->sort_tmp_bytes = 0;
     c->cand_cap = c->vstrips_cap = c->n_cand = c->n_vstrips = 0;
     dfree(c->d_panel_items);
+    dfree(c->d_short_list);
+    c->short_list_cap = c->n_short_list = 0;
+    c->use_short_list = false;
     dfree(c->d_fused_items);
     c->n_fused_items = c->fused_items_cap = 0;
     c->fused_items_valid = c->have_fused = false;
@@ -423,6 +431,14 @@ int env_int(const char *name, int fallback) {
     return e && *e ? atoi(e) : fallback;
 }
 
+// wavefronts of the short-row part of the AUTO launches: 64 entries of the entry list each, or
+// rpw consecutive rows each
+int64_t short_row_waves(const sddmm_ctx *c) {
+    if (c->rows_short <= 0) return 0;
+    if (c->use_short_list) return (c->n_short_list + WAVE - 1) / WAVE;
+    return ((int64_t)c->sM + c->rpw - 1) / c->rpw;
+}
+
 // Tiles and rows in one launch (k_auto_tiles); measured faster than two launches at
 // every row size the tile path takes (mixed-density shape: 23 -> 20 us at 128-byte
 // rows, 107 -> 92 us at 1 KiB rows).  Returns false when the layout has no fused
@@ -431,7 +447,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
     const Shape s = shape_of(c);
     if (c->tile_steps < 1 || c->tile_steps > env_int("SDDMM_FUSE_STEPS", 16) || !s.fullk || s.wide || s.unit == 1 || s.KU != 4 * c->tile_steps)
         return false;
-    const int64_t waves = c->rows_short > 0 ? ((int64_t)c->sM + c->rpw - 1) / c->rpw : 0;
+    const int64_t waves = short_row_waves(c);
     const int64_t short_blocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t tile_blocks = (c->n_windows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
@@ -448,7 +464,8 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
                                (const int32_t *)c->d_vrows, (const int32_t *)c->d_tile_cols,
                                (const TileDesc *)c->d_tiles, c->n_tiles,
                                (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows, c->nnz,
-                               tile_blocks, nblocks);
+                               tile_blocks, nblocks, (const int2 *)(c->use_short_list ? c->d_short_list : nullptr),
+                               c->n_short_list);
             launched = true;
         }
     });
@@ -457,7 +474,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
 
 void launch_auto(sddmm_ctx *c) {
     const Shape s = shape_of(c);
-    const int64_t waves = c->rows_short > 0 ? ((int64_t)c->sM + c->rpw - 1) / c->rpw : 0;
+    const int64_t waves = short_row_waves(c);
     const int64_t short_blocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t nblocks = short_blocks + item_blocks;
@@ -466,7 +483,8 @@ void launch_auto(sddmm_ctx *c) {
         SDDMM_LAUNCH(c, (k_auto<LT>), xcd_grid(nblocks), BLOCK,
                            (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
-                           c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks);
+                           c->dP, c->sM, c->ts, c->rpw, short_blocks, c->d_items, c->n_items, nblocks,
+                           (const int2 *)(c->use_short_list ? c->d_short_list : nullptr), c->n_short_list);
     });
 }
 
@@ -485,9 +503,11 @@ int classify_rows_count(sddmm_ctx *c, bool again = false) {
     if (nb > 0) {
         const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr, owner,
-                           c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc, 0);
+                           c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc, 0, c->d_short_sums);
         SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
+        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_short_sums, (int)nb,
+                           &c->d_pc->short_scanned);
         LAUNCH_CHECK(c);
     }
     return SDDMM_OK;
@@ -508,6 +528,22 @@ int classify_rows_items(sddmm_ctx *c) {
         SDDMM_LAUNCH(c, k_classify_write, nb, SCAN_BLOCK, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts, c->seg,
                            c->d_block_sums, c->d_items, 0);
+        LAUNCH_CHECK(c);
+    }
+    // the entries of the short rows as a list, taken 64 at a time (entry_list_body)
+    c->n_short_list = 0;
+    c->use_short_list = env_int("SDDMM_SHORT_LIST", 1) != 0 && c->rows_short > 0;
+    if (c->use_short_list) {
+        c->n_short_list = (int64_t)c->pc.nnz_short;
+        if (c->n_short_list > c->short_list_cap) {
+            dfree(c->d_short_list);
+            c->short_list_cap = 0;
+            ALLOC_TRY(c, c->d_short_list, (size_t)c->n_short_list * sizeof(int2));
+            c->short_list_cap = c->n_short_list;
+        }
+        SDDMM_LAUNCH(c, k_short_list_write, nb, SCAN_BLOCK, c->d_rowptr,
+                           (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts,
+                           (const unsigned int *)c->d_short_sums, c->d_short_list);
         LAUNCH_CHECK(c);
     }
     return SDDMM_OK;
@@ -986,7 +1022,11 @@ int do_plan(sddmm_ctx *c, int strategy) {
             // the rows nobody owns so far are classified in the same batch: most matrices have
             // no gathered strips, and their plan then waits for the device once
             c->ts = std::max(1, env_int("SDDMM_TS", 24));
-            c->seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+            // segment items of 256 entries: a wavefront walks its item chunk by chunk, one dependent
+            // round trip each, so a few long items set the duration of a short launch (eight rows of
+            // 554 entries as single items: 17.5 us on the mixed-density shape, 14.6 us in pieces of
+            // 256); on a matrix of 36 M entries pieces of 128..2048 differ by 3 %
+            c->seg = std::max(WAVE, env_int("SDDMM_SEG", 256));
             rc = classify_rows_count(c);
             if (rc) return rc;
             rc = fetch_counters(c);
@@ -1405,7 +1445,8 @@ static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
     c->n_fused_items = 0;
     if (nb > 0) {
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr,
-                           panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc, 2);
+                           panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc, 2,
+                           (unsigned int *)nullptr);
         SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
                            &c->d_pc->n_items);
         LAUNCH_CHECK(c);

@@ -546,10 +546,10 @@ def test_auto_row_classes_and_segments(engine_factory, monkeypatch):
     got, st = run_csr(engine_factory, rowptr, col, val, A, B, N, capi.AUTO)
     assert_parity(got, rowptr, col, val, A, B, what="auto classes")
     assert st.strategy_used == capi.AUTO and st.kernels_launched == 1
-    ts, seg = 24, 2048
+    ts, seg = 24, 256
     assert st.rows_short == np.count_nonzero((lens > 0) & (lens < ts))
     assert st.nnz_short == lens[lens < ts].sum()
-    assert st.rows_long == np.count_nonzero(lens > seg) == 1
+    assert st.rows_long == np.count_nonzero(lens > seg) >= 1
     assert st.rows_medium == np.count_nonzero((lens >= ts) & (lens <= seg))
     assert st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
     assert st.rows_nonempty == np.count_nonzero(lens)
