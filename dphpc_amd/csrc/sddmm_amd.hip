@@ -513,7 +513,7 @@ int classify_rows_count(sddmm_ctx *c, bool again = false) {
     return SDDMM_OK;
 }
 // ... and the items, once the counters are on the host (nothing may use the block sums in between)
-int classify_rows_items(sddmm_ctx *c) {
+int classify_rows_items(sddmm_ctx *c, bool with_short_list = true) {
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     c->n_items = (int64_t)c->pc.n_items;
     c->rows_short = (int64_t)c->pc.rows_short;
@@ -532,7 +532,7 @@ int classify_rows_items(sddmm_ctx *c) {
     }
     // the entries of the short rows as a list, taken 64 at a time (entry_list_body)
     c->n_short_list = 0;
-    c->use_short_list = env_int("SDDMM_SHORT_LIST", 1) != 0 && c->rows_short > 0;
+    c->use_short_list = with_short_list && env_int("SDDMM_SHORT_LIST", 1) != 0 && c->rows_short > 0;
     if (c->use_short_list) {
         c->n_short_list = (int64_t)c->pc.nnz_short;
         if (c->n_short_list > c->short_list_cap) {
@@ -1053,15 +1053,16 @@ int do_plan(sddmm_ctx *c, int strategy) {
                 rc = plan_tiles_fill(c);
                 if (rc) return rc;
             }
-            rc = classify_rows_items(c);
-            if (rc) return rc;
             // A matrix whose rows are short on average (fewer than 32 entries per non-empty
             // row), with no strip or panel taken, is a flat stream of entries: the flat
             // kernel (row index per entry, perfectly balanced) measured 6 % faster there than
             // the row split (power-law shape, K=32: 634 us against 672 us).
             const double avg_len = c->pc.rows_nonempty ? (double)c->nnz / (double)c->pc.rows_nonempty : 0.0;
-            if (resolved == SDDMM_AUTO && c->n_tiles == 0 && c->n_panel_items == 0 &&
-                avg_len < (double)env_int("SDDMM_FLAT_AVG", 32)) {
+            const bool flat = resolved == SDDMM_AUTO && c->n_tiles == 0 && c->n_panel_items == 0 &&
+                              avg_len < (double)env_int("SDDMM_FLAT_AVG", 32);
+            rc = classify_rows_items(c, !flat);      // (the flat kernel has no use for the entry list of the short rows)
+            if (rc) return rc;
+            if (flat) {
                 rc = ensure_rowidx(c);
                 if (rc) return rc;
                 resolved = SDDMM_FLAT;
