@@ -1161,22 +1161,46 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                       const TileWindow *__restrict__ win, int64_t n_win, int64_t nnz,
                                                       int64_t tile_blocks, int64_t nblocks,
-                                                      const int2 *__restrict__ short_list, int64_t n_short_list) {
+                                                      const int2 *__restrict__ short_list, int64_t n_short_list,
+                                                      int longest_first) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
-    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
-    if (blk < 0) return;
-    const int64_t tiles_before = blk * tile_blocks / nblocks;
-    if (((blk + 1) * tile_blocks / nblocks) != tiles_before) {
+    int64_t tile_block = -1, item_block = -1, short_block = -1;
+    if (longest_first) {
+        // Workgroups start in the order of their ids, round-robin over the XCDs: on every XCD the
+        // tile windows first (the longest wavefronts), then the segment items, then the chunks of
+        // the entry list, each XCD with its contiguous eighth of each kind.
+        const int x = (int)(blockIdx.x % NUM_XCD);
+        int64_t j = blockIdx.x / NUM_XCD;
+        const int64_t item_blocks = nblocks - tile_blocks - short_blocks;
+        const int64_t t_lo = x * tile_blocks / NUM_XCD, t_n = (x + 1) * tile_blocks / NUM_XCD - t_lo;
+        const int64_t i_lo = x * item_blocks / NUM_XCD, i_n = (x + 1) * item_blocks / NUM_XCD - i_lo;
+        const int64_t s_lo = x * short_blocks / NUM_XCD, s_n = (x + 1) * short_blocks / NUM_XCD - s_lo;
+        if (j < t_n) tile_block = t_lo + j;
+        else if ((j -= t_n) < i_n) item_block = i_lo + j;
+        else if ((j -= i_n) < s_n) short_block = s_lo + j;
+        else return;
+    } else {
+        const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+        if (blk < 0) return;
+        const int64_t tiles_before = blk * tile_blocks / nblocks;
+        if (((blk + 1) * tile_blocks / nblocks) != tiles_before) {
+            tile_block = tiles_before;
+        } else {
+            const int64_t rb = blk - tiles_before, rest = nblocks - tile_blocks;
+            const int64_t item_blocks = rest - short_blocks;
+            const int64_t items_before = rb * item_blocks / rest;
+            if (((rb + 1) * item_blocks / rest) != items_before) item_block = items_before;
+            else short_block = rb - items_before;
+        }
+    }
+    if (tile_block >= 0) {
         tile_window_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
-                                          tiles_before * WAVES_PER_BLOCK + wave_in_block(),
+                                          tile_block * WAVES_PER_BLOCK + wave_in_block(),
                                           win_lds[wave_in_block()]);
         return;
     }
-    const int64_t rb = blk - tiles_before, rest = nblocks - tile_blocks;
-    const int64_t item_blocks = rest - short_blocks;
-    const int64_t items_before = rb * item_blocks / rest;
-    if (((rb + 1) * item_blocks / rest) != items_before) {
-        const int64_t w = items_before * WAVES_PER_BLOCK + wave_in_block();
+    if (item_block >= 0) {
+        const int64_t w = item_block * WAVES_PER_BLOCK + wave_in_block();
         if (w >= n_items) return;
         const RowItem it = items[w];
         const int row = __builtin_amdgcn_readfirstlane(it.row);
@@ -1184,7 +1208,7 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
         const int end = __builtin_amdgcn_readfirstlane(it.end);
         row_segment_body<L>(A, B, KU, col, sval, P, row, start, end, lane_id());
     } else {
-        const int64_t sb = rb - items_before;
+        const int64_t sb = short_block;
         if (short_list) {
             entry_list_body<L>(A, B, KU, short_list, n_short_list, col, sval, P, sb * WAVES_PER_BLOCK + wave_in_block(),
                                lane_id());

@@ -452,12 +452,20 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
     const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t tile_blocks = (c->n_windows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t nblocks = short_blocks + item_blocks + tile_blocks;
+    // Order of the blocks on every XCD.  Rows of up to 128 bytes: the tile windows (the wavefronts that
+    // live longest) start first, then the items, then the chunks of the entry list -- measured
+    // 14.7 -> 13.5 us on the mixed-density shape; at 256 bytes it makes no difference, at 1 KiB,
+    // where the gathers of the short rows are the longer half, the even deal is 3 % faster.
+    const int longest_first = env_int("SDDMM_LONGEST_FIRST", c->tile_steps <= 2 ? 1 : 0);
+    auto eighth = [](int64_t n) { return (n + NUM_XCD - 1) / NUM_XCD; };
+    const int64_t grid = longest_first ? NUM_XCD * (eighth(short_blocks) + eighth(item_blocks) + eighth(tile_blocks))
+                                       : xcd_grid(nblocks);
     bool launched = false;
     with_layout(s, [&](auto L) {
         using LT = decltype(L);
         constexpr int KU_ = LT::LPN * LT::UPL;
         if constexpr (!LT::LONG && LT::FULLK && !LT::WIDE && LT::U::ELEMS > 1 && (KU_ == 4 || KU_ == 8 || KU_ == 16 || KU_ == 32 || KU_ == 64)) {
-            SDDMM_LAUNCH(c, (k_auto_tiles<LT, KU_ / 4>), xcd_grid(nblocks), BLOCK,
+            SDDMM_LAUNCH(c, (k_auto_tiles<LT, KU_ / 4>), grid, BLOCK,
                                (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr,
                                (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->d_col, c->d_sval,
                                c->dP, c->sM, c->N, c->ts, c->rpw, short_blocks, c->d_items, c->n_items,
@@ -465,7 +473,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
                                (const TileDesc *)c->d_tiles, c->n_tiles,
                                (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows, c->nnz,
                                tile_blocks, nblocks, (const int2 *)(c->use_short_list ? c->d_short_list : nullptr),
-                               c->n_short_list);
+                               c->n_short_list, longest_first);
             launched = true;
         }
     });
