@@ -543,6 +543,8 @@ int classify_rows_items(sddmm_ctx *c, bool with_short_list = true) {
     c->use_short_list = with_short_list && env_int("SDDMM_SHORT_LIST", 1) != 0 && c->rows_short > 0;
     if (c->use_short_list) {
         c->n_short_list = (int64_t)c->pc.nnz_short;
+        if ((int64_t)c->raw.short_scanned != c->n_short_list)
+            return fail(c, SDDMM_ERR_HIP, "internal: scan of the short rows disagrees with their entry count");
         if (c->n_short_list > c->short_list_cap) {
             dfree(c->d_short_list);
             c->short_list_cap = 0;
