@@ -63,6 +63,31 @@ def test_full_size(engine_factory, name, K, other):
     e.close()
 
 
+@pytest.mark.parametrize("name,K", [("fem_banded", 32), ("fem_banded", 128), ("mixed_density", 64)])
+def test_fused_full_size(engine_factory, name, K):
+    """SDDMM followed by SpMM at the benchmark's sizes: the panel kernel (fem_banded) and the
+    gather kernels (mixed_density) against the oracle, and the row sums of O against float64."""
+    w = W.make(name, "full", K=K)
+    print("fused full size", name, K, "nnz", w.nnz, flush=True)
+    e = engine_factory()
+    e.set_dense(w.A, w.B)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    e.plan(capi.AUTO)
+    got_o = e.run_fused()
+    got_p = e.values()
+    ref_p, ref_o = O.fusedmm_csr(w.rowptr, w.col, w.sval, w.A, w.B)
+    _, mag_p = O.sddmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+    o64, mag_o = O.fusedmm_csr_f64(w.rowptr, w.col, w.sval, w.A, w.B)
+    ok, worst, i = O.check_values(got_p, ref_p, mag=mag_p)
+    assert ok, (name, K, "P", i, worst)
+    ok, worst, i = O.check_values(got_o[:w.M].ravel(), ref_o.ravel(), mag=mag_o.ravel())
+    assert ok, (name, K, "O", i, worst)
+    assert abs(got_o[:w.M].astype(np.float64).sum() - o64.sum()) <= 1e-5 * mag_o.sum()
+    if name == "fem_banded":
+        assert e.stats().kernels_launched == 1        # every row belongs to a panel
+    e.close()
+
+
 def test_positions_beyond_2_to_the_30(engine_factory):
     """1.2e9 stored entries: positions above 2^30, byte offsets above 4 GiB in the entry
     arrays.  Groups of 8 identical rows, so AUTO takes the panel kernel; the exact kernel
