@@ -1348,12 +1348,15 @@ constexpr int panel_mfma_waves(int steps) { return steps <= 4 ? 2 : 4; }
 constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;   // rotation by 4 / 8 lanes inside every row of 16
 constexpr int PANEL_TILE_PITCH = 48;                        // floats per row of the P tile: conflict-free 4-byte reads
 
+// waves per SIMD the register allocation aims at: the fused kernel keeps 32 * STEPS accumulators of
+// the output rows (3 waves at 128-byte rows -- 4 were no faster --, 2 at 256 bytes, measured 89 us
+// against 114 us with 1; at 512 bytes the accumulators leave room for one)
+constexpr int panel_mfma_min_waves(int steps, bool fused) {
+    return fused ? (steps == 2 ? 3 : steps == 4 ? 2 : 1) : steps == 8 ? 4 : 1;
+}
+
 template <int DT, int STEPS, bool FUSED = false>
-#ifndef SDDMM_FUSED_OCC2
-#define SDDMM_FUSED_OCC2 3
-#define SDDMM_FUSED_OCC4 2
-#endif
-__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, FUSED ? (STEPS == 2 ? SDDMM_FUSED_OCC2 : STEPS == 4 ? SDDMM_FUSED_OCC4 : 1) : STEPS == 8 ? 4 : 1) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_waves(STEPS, FUSED)) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const float *__restrict__ sval, float *__restrict__ P,
@@ -1384,10 +1387,7 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, FUSED ? (STEPS == 2
                 : 16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
     constexpr int ROW_UNITS = STEPS * 4;
     // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
-#ifndef SDDMM_FUSED_GROUPS
-#define SDDMM_FUSED_GROUPS 4
-#endif
-    constexpr int GROUPS = STEPS >= 8 ? 2 : FUSED ? SDDMM_FUSED_GROUPS : 4;
+    constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
     const uint4 *__restrict__ Au = (const uint4 *)A;
     const uint4 *__restrict__ Bu = (const uint4 *)B;
     constexpr int A_REGS = BLOCKS ? STEPS / 2 : STEPS;
