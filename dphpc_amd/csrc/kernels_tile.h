@@ -981,8 +981,10 @@ __device__ __forceinline__ void tile_window_wave(const void *__restrict__ A, con
                                                  const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                  const TileWindow *__restrict__ win, int64_t n_win,
                                                  const int32_t *__restrict__ col, const float *__restrict__ sval,
-                                                 float *__restrict__ P, int64_t nnz, int64_t w, float *lds) {
+                                                 float *__restrict__ P, int64_t nnz, int64_t w, float *lds,
+                                                 const int32_t *__restrict__ order = nullptr) {
     if (w >= n_win) return;
+    if (order) w = order[w];                              // the plan's order of the windows (k_window_order)
     const int lane = lane_id();
     if (win == nullptr) {                                 // the plan chose the tile-by-tile walk for this matrix
         tile_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, TILE_WINDOW, sval, P, w);
@@ -1132,12 +1134,58 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
                                                 const TileDesc *__restrict__ tiles, int64_t n_tiles,
                                                 const TileWindow *__restrict__ win, int64_t n_win,
                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
-                                                float *__restrict__ P, int64_t nnz, int64_t nblocks) {
+                                                float *__restrict__ P, int64_t nnz, int64_t nblocks,
+                                                const int32_t *__restrict__ order) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
     tile_window_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
-                                blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()]);
+                                blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()], order);
+}
+
+// Order of the windows for operands that exceed an XCD's L2.  The launch gives every XCD a
+// contiguous eighth of the logical windows (xcd_remap); sorted by the key below, that eighth is
+// one block of a RB x CB grid over (strip rows, tile columns), RB * CB = 8, walked by finer
+// column slices: the XCD keeps its part of A resident and streams through its part of B once,
+// instead of touching all of B from every strip (the storage order of the descriptors).
+// Counting sort in three launches: histogram, scan of the WINDOW_BINS counters, scatter (the
+// order inside a bin is whatever the atomics give; every entry is computed on its own, so the
+// result does not depend on it).
+constexpr int WINDOW_SLICES = 8;                      // column slices inside a block
+constexpr int WINDOW_BINS = NUM_XCD * WINDOW_SLICES;
+__device__ __forceinline__ int window_bin(const TileDesc *__restrict__ tiles, int64_t w, int64_t strip_span,
+                                          int64_t tile_col_span, int RB, int CB) {
+    const int4 h = *reinterpret_cast<const int4 *>(tiles + w * TILE_WINDOW);        // strip, tj, ..
+    int64_t strip = h.x >= GATHERED_BASE ? h.x - GATHERED_BASE : h.x;
+    strip = strip < strip_span ? strip : strip_span - 1;
+    int64_t tj = h.y < 0 ? 0 : h.y;
+    tj = tj < tile_col_span ? tj : tile_col_span - 1;
+    const int rb = (int)(strip * RB / strip_span);
+    const int fine = (int)(tj * (CB * WINDOW_SLICES) / tile_col_span);               // cb * WINDOW_SLICES + slice
+    return rb * (CB * WINDOW_SLICES) + fine;
+}
+__global__ __launch_bounds__(256) void k_window_histogram(const TileDesc *__restrict__ tiles, int64_t n_win,
+                                                          int64_t strip_span, int64_t tile_col_span, int RB, int CB,
+                                                          unsigned int *__restrict__ bins) {
+    const int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (w < n_win) atomicAdd(&bins[window_bin(tiles, w, strip_span, tile_col_span, RB, CB)], 1u);
+}
+// one workgroup of WINDOW_BINS threads: counts -> start positions (also the scatter's cursors)
+__global__ __launch_bounds__(WINDOW_BINS) void k_window_offsets(unsigned int *__restrict__ bins) {
+    __shared__ unsigned int v[WINDOW_BINS];
+    v[threadIdx.x] = bins[threadIdx.x];
+    __syncthreads();
+    unsigned int before = 0;
+    for (int i = 0; i < (int)threadIdx.x; ++i) before += v[i];
+    bins[threadIdx.x] = before;
+}
+__global__ __launch_bounds__(256) void k_window_scatter(const TileDesc *__restrict__ tiles, int64_t n_win,
+                                                        int64_t strip_span, int64_t tile_col_span, int RB, int CB,
+                                                        unsigned int *__restrict__ cursors, int32_t *__restrict__ order) {
+    const int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (w >= n_win) return;
+    const unsigned int at = atomicAdd(&cursors[window_bin(tiles, w, strip_span, tile_col_span, RB, CB)], 1u);
+    order[at] = (int32_t)w;
 }
 
 // AUTO in one launch when a matrix has tiles and rows: logical blocks are dealt out
@@ -1162,7 +1210,7 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
                                                       const TileWindow *__restrict__ win, int64_t n_win, int64_t nnz,
                                                       int64_t tile_blocks, int64_t nblocks,
                                                       const int2 *__restrict__ short_list, int64_t n_short_list,
-                                                      int longest_first) {
+                                                      int longest_first, const int32_t *__restrict__ order) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     int64_t tile_block = -1, item_block = -1, short_block = -1;
     if (longest_first) {
@@ -1196,7 +1244,7 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_a
     if (tile_block >= 0) {
         tile_window_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
                                           tile_block * WAVES_PER_BLOCK + wave_in_block(),
-                                          win_lds[wave_in_block()]);
+                                          win_lds[wave_in_block()], order);
         return;
     }
     if (item_block >= 0) {

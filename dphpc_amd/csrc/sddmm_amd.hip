@@ -75,6 +75,10 @@ struct sddmm_ctx {
     int64_t n_tiles = 0, tiles_cap = 0, nnz_tiles = 0;
     int tile_steps = 0;
     bool tiles_active = false;       // d_tiles describes the current pattern
+    int32_t *d_win_order = nullptr;  // order in which the launch takes the windows (null: storage order)
+    unsigned int *d_win_bins = nullptr;
+    int64_t win_order_cap = 0;
+    bool use_win_order = false;
     TileWindow *d_windows = nullptr; // one record per TILE_WINDOW consecutive descriptors
     int64_t n_windows = 0, windows_cap = 0;
     bool use_windows = false;        // tile kernels take windows as batches (else they walk them tile by tile)
@@ -262,6 +266,10 @@ void release_sparse(sddmm_ctx *c) {
     dfree(c->d_tiles);
     dfree(c->d_tile_cols);
     dfree(c->d_windows);
+    dfree(c->d_win_order);
+    dfree(c->d_win_bins);
+    c->win_order_cap = 0;
+    c->use_win_order = false;
     c->n_windows = c->windows_cap = 0;
     c->ustrips_cap = 0;
     dfree(c->d_sort_tmp);
@@ -473,7 +481,8 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
                                (const TileDesc *)c->d_tiles, c->n_tiles,
                                (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows, c->nnz,
                                tile_blocks, nblocks, (const int2 *)(c->use_short_list ? c->d_short_list : nullptr),
-                               c->n_short_list, longest_first);
+                               c->n_short_list, longest_first,
+                               (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr));
             launched = true;
         }
     });
@@ -701,6 +710,51 @@ int plan_gathered_take(sddmm_ctx *c) {
     return SDDMM_OK;
 }
 
+// When the storage order of the windows (strip by strip) makes every XCD touch more of A and B
+// than its L2 holds, the launch takes them block by block of a RB x CB grid over (strips, tile
+// columns), one block per XCD (k_window_histogram and following).
+int plan_window_order(sddmm_ctx *c) {
+    c->use_win_order = false;
+    const int mode = env_int("SDDMM_WINDOW_ORDER", -1);          // -1: decide here, 0: never, 1: always
+    const double row_bytes = (double)c->K * (double)elem_size(c->dtype);
+    const double a_bytes = (double)c->sM * row_bytes, b_bytes = (double)c->N * row_bytes;
+    const double l2 = 4.0 * 1024 * 1024;
+    // storage order: an XCD has an eighth of the strips and, over the launch, all of B
+    if (mode == 0 || c->n_windows < 8 * NUM_XCD) return SDDMM_OK;
+    // (gathered strips come sorted by column window already: reordering them measured 12 % slower)
+    if (mode < 0 && c->n_tiles != c->n_tiles_natural) return SDDMM_OK;
+    if (mode < 0 && a_bytes / NUM_XCD + b_bytes <= 0.75 * l2) return SDDMM_OK;
+    // resident part of A per XCD within half an L2, then the least traffic A * CB + B * RB
+    int RB = NUM_XCD, CB = 1;
+    double best = -1.0;
+    for (int rb = 1; rb <= NUM_XCD; rb *= 2) {
+        const int cb = NUM_XCD / rb;
+        const double traffic = a_bytes * cb + b_bytes * rb;
+        const bool fits = a_bytes / rb <= 0.6 * l2;
+        if (!fits && rb != NUM_XCD) continue;
+        if (best < 0 || traffic < best) { best = traffic; RB = rb; CB = cb; }
+    }
+    if (c->n_windows > c->win_order_cap) {
+        dfree(c->d_win_order);
+        c->win_order_cap = 0;
+        ALLOC_TRY(c, c->d_win_order, (size_t)c->n_windows * sizeof(int32_t));
+        c->win_order_cap = c->n_windows;
+    }
+    if (!c->d_win_bins) ALLOC_TRY(c, c->d_win_bins, (size_t)WINDOW_BINS * sizeof(unsigned int));
+    HIP_TRY(c, hipMemsetAsync(c->d_win_bins, 0, (size_t)WINDOW_BINS * sizeof(unsigned int), c->stream));
+    const int64_t strip_span = std::max<int64_t>(1, std::max(((int64_t)c->sM + 15) / 16, c->n_vstrips));
+    const int64_t tile_col_span = std::max<int64_t>(1, ((int64_t)c->N + 15) / 16);
+    const unsigned grid = (unsigned)((c->n_windows + 255) / 256);
+    SDDMM_LAUNCH(c, k_window_histogram, grid, 256, (const TileDesc *)c->d_tiles, c->n_windows, strip_span, tile_col_span,
+                       RB, CB, c->d_win_bins);
+    SDDMM_LAUNCH(c, k_window_offsets, 1, WINDOW_BINS, c->d_win_bins);
+    SDDMM_LAUNCH(c, k_window_scatter, grid, 256, (const TileDesc *)c->d_tiles, c->n_windows, strip_span, tile_col_span,
+                       RB, CB, c->d_win_bins, c->d_win_order);
+    LAUNCH_CHECK(c);
+    c->use_win_order = true;
+    return SDDMM_OK;
+}
+
 int plan_tiles_fill(sddmm_ctx *c) {
     if (c->n_tiles == 0) return SDDMM_OK;
     if (c->n_tiles > c->tiles_cap) {
@@ -742,6 +796,10 @@ int plan_tiles_fill(sddmm_ctx *c) {
     // tiles are sparsely filled; tile by tile from the descriptors' masks where they are nearly
     // full (measured: 92 entries per tile 12.8 -> 11.3 us as batches, 256 per tile 8.5 -> 9.4 us)
     c->n_windows = (c->n_tiles + TILE_WINDOW - 1) / TILE_WINDOW;
+    {
+        const int rc = plan_window_order(c);
+        if (rc) return rc;
+    }
     c->use_windows = c->nnz_tiles < (int64_t)env_int("SDDMM_WINDOW_FILL", 176) * c->n_tiles;
     if (!c->use_windows) {
         c->tiles_active = true;
@@ -875,7 +933,8 @@ void launch_tile_t(sddmm_ctx *c) {
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
                        (const int32_t *)c->d_tile_cols, (const TileDesc *)c->d_tiles, c->n_tiles,
                        (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows,
-                       (const int32_t *)c->d_col, (const float *)c->d_sval, c->dP, c->nnz, nblocks);
+                       (const int32_t *)c->d_col, (const float *)c->d_sval, c->dP, c->nnz, nblocks,
+                       (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr));
 }
 template <int DT>
 void launch_tile_steps(sddmm_ctx *c) {

@@ -932,3 +932,30 @@ def test_tile_windows_and_tile_walk_agree_with_the_oracle(engine_factory, monkey
     got, st = run_csr(engine_factory, rowptr, col, val, Ab, Bb, N, capi.MFMA_TILE, dtype)
     assert st.nnz_mfma == len(col) and st.mfma_tiles > 0
     assert_parity(got, rowptr, col, val, A, B, what="tiles K=%d limit %s" % (K, fill_limit))
+
+
+@pytest.mark.parametrize("fill_limit", ["0", "100000"])
+@pytest.mark.parametrize("name,K", [("dense_tiles", 128), ("dense_tiles", 512), ("mixed_density", 64)])
+def test_windows_taken_block_by_block_over_strips_and_columns(engine_factory, monkeypatch, name, K, fill_limit):
+    """The plan may hand the windows to the launch in an order of its own (blocks of strips x tile
+    columns, one per XCD, for operands that exceed an L2).  Forced here on small inputs, for the
+    batch and the tile-by-tile form of the windows, with and without row kernels in the same
+    launch: every entry is still computed exactly once."""
+    monkeypatch.setenv("SDDMM_WINDOW_ORDER", "1")
+    monkeypatch.setenv("SDDMM_WINDOW_FILL", fill_limit)
+    w = W.make(name, "small", K=K)
+    bf16 = w.dtype == "bf16"
+    e = engine_factory()
+    if bf16:
+        e.set_dense(w.A_bits, w.B_bits, capi.BF16)
+    else:
+        e.set_dense(w.A, w.B)
+    for strategy in (capi.AUTO, capi.MFMA_TILE):
+        e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)      # clears P
+        e.plan(strategy)
+        e.run()
+        st = e.stats()
+        assert st.mfma_tiles > 0
+        assert_parity(e.values(), w.rowptr, w.col, w.sval, w.A, w.B, what="%s K=%d ordered windows" % (name, K))
+        assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == w.nnz
+    e.close()
