@@ -1504,25 +1504,47 @@ int sddmm_run(sddmm_ctx *c) {
 // items of the fused kernel: the rows of more than FUSED_ROW_MAX entries, cut into segments of SDDMM_SEG entries
 static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
     if (c->fused_items_valid && c->fused_items_panels == (panel_owner != nullptr)) return SDDMM_OK;
-    const int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+    int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     const int arc = ensure_arena(c);
     if (arc) return arc;
     ARENA_HOLDS(c, nb, c->block_sums_cap, "block sums");
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
-                              sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
-    HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
     c->n_fused_items = 0;
     if (nb > 0) {
-        SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr,
-                           panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc, 2,
-                           (unsigned int *)nullptr);
-        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
-                           &c->d_pc->n_items);
-        LAUNCH_CHECK(c);
         DevCounters tmp;
-        HIP_TRY(c, hipMemcpyAsync(&tmp, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
-        HIP_TRY(c, hipStreamSynchronize(c->stream));
+        auto count = [&]() -> int {
+            HIP_TRY(c, hipMemsetAsync(&c->d_pc->k[K_ROWS_SHORT][0], 0,
+                                      sizeof(unsigned long long) * SPREAD * (K_NNZ_LONG - K_ROWS_SHORT + 1), c->stream));
+            HIP_TRY(c, hipMemsetAsync(&c->d_pc->n_items, 0, sizeof(unsigned long long), c->stream));
+            SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr,
+                               panel_owner, c->sM, FUSED_ROW_MAX + 1, seg, c->d_block_sums, c->d_pc, 2,
+                               (unsigned int *)nullptr);
+            SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
+                               &c->d_pc->n_items);
+            LAUNCH_CHECK(c);
+            HIP_TRY(c, hipMemcpyAsync(&tmp, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
+            HIP_TRY(c, hipStreamSynchronize(c->stream));
+            return SDDMM_OK;
+        };
+        int rc = count();
+        if (rc) return rc;
+        // Few long rows: one wavefront per row walks its chunks one after the other and the launch
+        // waits for them (3 000 rows of 554 entries: 50 us as single items, 42 us in pieces of 256,
+        // the pieces of a row adding to O atomically).  With enough items to fill the chip several
+        // times the long segments stay: there the atomic adds cost more than they return.
+        const PlanCounters first = summarize(tmp);
+        const int64_t item_entries = (int64_t)(first.nnz_medium + first.nnz_long);
+        // (rows of up to 128 bytes; at 256 bytes it changes nothing, at 1 KiB the adds of 256 floats per piece lose 4 %)
+        if ((int64_t)tmp.n_items > 0 && (int64_t)tmp.n_items < 4096 && !getenv("SDDMM_SEG") &&
+            (size_t)c->K * elem_size(c->dtype) <= 128) {
+            int shorter = (int)std::min<int64_t>(seg, ((item_entries / 8192 + WAVE - 1) / WAVE) * WAVE);
+            shorter = std::max(shorter, 256);
+            if (shorter < seg) {
+                seg = shorter;
+                rc = count();
+                if (rc) return rc;
+            }
+        }
         c->n_fused_items = (int64_t)tmp.n_items;
         if (c->n_fused_items > c->fused_items_cap) {
             dfree(c->d_fused_items);
