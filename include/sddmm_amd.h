@@ -218,8 +218,9 @@ int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, cons
  * (src/competitors/cpu/cpu_basic.hpp:18-51).  O is M x K fp32 row-major, owned by the
  * context.  Needs K <= 256, a multiple of 4 (fp32 operands) or 8 (bf16, fp16), and
  * row-sorted entries (CSR, or COO with non-decreasing rows); SDDMM_ERR_UNSUPPORTED otherwise.
- * Rows longer than 2048 entries are accumulated with atomic adds, so their last bits
- * may differ from run to run.
+ * Rows cut into several work items (longer than 2048 entries; longer than 256 where a
+ * matrix of rows of up to 128 bytes has only a few thousand such rows) are accumulated
+ * with atomic adds, so their last bits may differ from run to run.
  * fp32 operands with K = 32, 64 or 128: the rows that the current plan (SDDMM_AUTO is planned
  * if there is none) runs as 8-row panels take a matrix-core kernel that shares every
  * gathered B row between the 8 rows and between both products; panels whose column list
