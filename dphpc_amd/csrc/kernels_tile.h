@@ -1041,7 +1041,9 @@ __device__ __forceinline__ void tile_window_wave(const void *__restrict__ A, con
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) dst[s] = src[s * 4];
     };
-    constexpr bool ALL_B = STEPS <= 4;                    // rows of up to 256 bytes: the B rows of all four tiles in flight
+    // rows of up to 128 bytes: the B rows of all four tiles in flight; longer rows two tiles at a time (at 256
+    // bytes four in flight cost 13 registers and a wave per SIMD of the launch that also runs rows: 22.0 -> 21.2 us)
+    constexpr bool ALL_B = STEPS <= 2;
     uint4 b[ALL_B ? TILE_WINDOW : 2][STEPS];
     if constexpr (ALL_B) {
 #pragma unroll
@@ -1197,7 +1199,7 @@ __global__ __launch_bounds__(256) void k_window_scatter(const TileDesc *__restri
 #define SDDMM_FUSED_WAVES 6
 #endif
 template <class L, int STEPS>
-__global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : 1) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
+__global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : STEPS == 4 ? 5 : 1) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                       const int32_t *__restrict__ rowptr,
                                                       const unsigned char *__restrict__ owner,
                                                       const int32_t *__restrict__ col,
