@@ -460,11 +460,11 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
     const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t tile_blocks = (c->n_windows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t nblocks = short_blocks + item_blocks + tile_blocks;
-    // Order of the blocks on every XCD.  Rows of up to 128 bytes: the tile windows (the wavefronts that
+    // Order of the blocks on every XCD.  Rows of up to 256 bytes: the tile windows (the wavefronts that
     // live longest) start first, then the items, then the chunks of the entry list -- measured
-    // 14.7 -> 13.5 us on the mixed-density shape; at 256 bytes it makes no difference, at 1 KiB,
-    // where the gathers of the short rows are the longer half, the even deal is 3 % faster.
-    const int longest_first = env_int("SDDMM_LONGEST_FIRST", c->tile_steps <= 2 ? 1 : 0);
+    // 14.7 -> 13.5 us on the mixed-density shape at 128 bytes, 21.3 -> 21.1 us (cold 29.7 -> 27.8) at
+    // 256; at 1 KiB, where the gathers of the short rows are the longer half, the even deal is 3 % faster.
+    const int longest_first = env_int("SDDMM_LONGEST_FIRST", c->tile_steps <= 4 ? 1 : 0);
     auto eighth = [](int64_t n) { return (n + NUM_XCD - 1) / NUM_XCD; };
     const int64_t grid = longest_first ? NUM_XCD * (eighth(short_blocks) + eighth(item_blocks) + eighth(tile_blocks))
                                        : xcd_grid(nblocks);
