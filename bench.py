@@ -101,17 +101,23 @@ class Checker:
         return ok, worst, i
 
 
-def load_traffic(key):
-    """HBM bytes per launch from an earlier rocprofv3 --pmc pair of runs (FETCH_SIZE,
-    WRITE_SIZE), recorded by hand in profiles/traffic.json: a constant of the
-    repository, NOT measured by this run; None when there is no record."""
+def load_traffic(key, field="bytes_per_launch"):
+    """HBM bytes per launch (or another recorded field: `l2_hit`, `bound`) from an
+    earlier rocprofv3 --pmc pair of runs (FETCH_SIZE, WRITE_SIZE), recorded by hand in
+    profiles/traffic.json: a constant of the repository, NOT measured by this run;
+    None when there is no record."""
     p = os.path.join(ROOT, "profiles", "traffic.json")
     if not os.path.exists(p):
         return None
     try:
-        return json.load(open(p)).get(key, {}).get("bytes_per_launch")
+        return json.load(open(p)).get(key, {}).get(field)
     except Exception:
         return None
+
+
+TRAFFIC_SOURCE = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (and TCC hits / requests) of an "
+                  "earlier run of this command, recorded constants, not measured by this run")
+SINGLE_KERNEL = ["FLAT", "ROW_WAVE", "SHORT_ROWS"]     # strategies that are one gather kernel, none of AUTO's parts
 
 
 # --------------------------------------------------------------------------- GPU side
@@ -237,11 +243,21 @@ def fused_leg(e, w, capi, reps, check):
 
 
 def fractions(w, us, cold_us):
-    """Compulsory bytes over launch time against the HBM peak (and the dense-tile
-    shape's flops against the bf16 MFMA peak)."""
+    """Compulsory bytes over launch time against the HBM peak.  `frac` is taken from the
+    cold launches, the only ones whose operands come from HBM; `frac_llc` from the
+    launches of a loop, which find a working set below 256 MB in the last-level cache.
+    Also the recorded counter figures of the shape (traffic against the peak, L2 hit
+    rate, what bounds it) and, for 16-bit operands, the flops against the bf16 MFMA peak."""
     comp = w.bytes_compulsory()
-    d = {"frac": comp / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-         "frac_cold": None if not cold_us else comp / (cold_us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    d = {"frac": None if not cold_us else comp / (cold_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+         "frac_llc": comp / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    key = "%s_K%d_%s" % (w.name, w.K, w.dtype)
+    traffic = load_traffic(key)
+    d["traffic"] = traffic
+    d["traffic_frac"] = None if not (traffic and cold_us) else traffic / (cold_us * 1e-6) / 1e9 / HBM_PEAK_GBS
+    d["traffic_frac_llc"] = None if not traffic else traffic / (us * 1e-6) / 1e9 / HBM_PEAK_GBS
+    d["l2_hit"] = load_traffic(key, "l2_hit")
+    d["bound"] = load_traffic(key, "bound")
     if w.dtype != "f32":
         d["mfma_frac"] = w.flops() / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS
     return d
@@ -259,6 +275,8 @@ def per_config_entry(name, K, capi, workloads, steps, warmup, flusher, no_cpu, s
     ran = {s: r for s, r in fixed.items() if "us" in r}
     best = min(ran, key=lambda s: ran[s]["us"])
     best_cold = min(ran, key=lambda s: ran[s]["cold_us"] or float("inf"))
+    single = [s for s in SINGLE_KERNEL if s in ran]
+    best_single = min(single, key=lambda s: ran[s]["us"])
     entry = {
         "workload": w.name, "K": w.K, "dtype": w.dtype, "M": w.M, "N": w.N, "nnz": w.nnz,
         "auto_us": auto["us"], "auto_cold_us": auto["cold_us"], "auto_resolved": auto["resolved"],
@@ -266,6 +284,8 @@ def per_config_entry(name, K, capi, workloads, steps, warmup, flusher, no_cpu, s
         "best_fixed": best, "best_fixed_us": ran[best]["us"],
         "best_fixed_cold": best_cold, "best_fixed_cold_us": ran[best_cold]["cold_us"],
         "auto_over_best_fixed": ran[best]["us"] / auto["us"],
+        "best_single_kernel": best_single, "best_single_kernel_us": ran[best_single]["us"],
+        "auto_over_best_single_kernel": ran[best_single]["us"] / auto["us"],
         "fixed_us": {s: (round(r["us"], 2) if "us" in r else r["error"]) for s, r in fixed.items()},
         "gflops": w.flops() / (auto["us"] * 1e-6) / 1e9,
         "bytes_compulsory": w.bytes_compulsory(),
@@ -284,9 +304,11 @@ def per_config_entry(name, K, capi, workloads, steps, warmup, flusher, no_cpu, s
         entry["cpu_allcores_gflops"] = round(allc["value"], 2)
         entry["cpu_cores"] = allc["cores"]
         entry["cpu_sample"] = base["sample"]
-    log("per_config %s K=%d: AUTO %.1f us (cold %s), best fixed %s %.1f us, frac %.3f  [%.1fs]" % (
-        w.name, w.K, auto["us"], "%.1f" % auto["cold_us"] if auto["cold_us"] else "-", best, ran[best]["us"],
-        entry["frac"], time.time() - t0))
+    log("per_config %s K=%d: AUTO %.1f us (cold %s), plan %.0f us, best fixed %s %.1f us, best single kernel %s %.1f us, "
+        "frac %s (llc %.3f)  [%.1fs]" % (
+            w.name, w.K, auto["us"], "%.1f" % auto["cold_us"] if auto["cold_us"] else "-", auto["plan_us"], best,
+            ran[best]["us"], best_single, ran[best_single]["us"],
+            "%.3f" % entry["frac"] if entry["frac"] else "-", entry["frac_llc"], time.time() - t0))
     return entry
 
 
@@ -378,22 +400,29 @@ def main():
     ev_plan = e.time_runs(1, 5, include_plan=True)
     st = e.stats()
     flops, gathered, compulsory = w.flops(), w.bytes_gathered(), w.bytes_compulsory()
-    achieved = compulsory / (ev_avg * 1e-3) / 1e9
-    achieved_cold = None if not ev_cold else compulsory / (ev_cold * 1e-3) / 1e9
-    traffic = load_traffic("%s_K%d_%s" % (w.name, w.K, w.dtype))
+    # The HBM figure comes from the cold launches: in the loop a working set below 256 MB is
+    # served by the last-level cache, which `achieved_llc` / `frac_llc` report apart.  Only
+    # with --include-plan (no cold launches are timed then) does the loop stand in.
+    achieved_llc = compulsory / (ev_avg * 1e-3) / 1e9
+    hbm_ms = ev_cold if ev_cold else ev_avg
+    achieved = compulsory / (hbm_ms * 1e-3) / 1e9
+    key = "%s_K%d_%s" % (w.name, w.K, w.dtype)
+    traffic = load_traffic(key)
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS,
+                "launches": "cold: each follows a 1 GiB device copy, operands come from HBM" if ev_cold else
+                "in a loop (no cold launches were timed): the last-level cache may serve them",
                 "bytes": "compulsory: every operand byte once per launch",
-                "achieved_cold": achieved_cold,
-                "frac_cold": None if achieved_cold is None else achieved_cold / HBM_PEAK_GBS,
+                "achieved_llc": achieved_llc,
+                "frac_llc": achieved_llc / HBM_PEAK_GBS,
                 "gathered_equiv_gbs": gathered / (ev_avg * 1e-3) / 1e9,
                 "traffic": traffic,
-                "traffic_source": None if traffic is None else
-                "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this "
-                "command, a recorded constant, not measured by this run"}
+                "traffic_source": None if traffic is None else TRAFFIC_SOURCE,
+                "l2_hit": load_traffic(key, "l2_hit"),
+                "limit": load_traffic(key, "bound")}
     if traffic:
-        roofline["traffic_frac"] = traffic / (ev_avg * 1e-3) / 1e9 / HBM_PEAK_GBS
-        roofline["traffic_frac_cold"] = None if not ev_cold else traffic / (ev_cold * 1e-3) / 1e9 / HBM_PEAK_GBS
+        roofline["traffic_frac"] = traffic / (hbm_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        roofline["traffic_frac_llc"] = traffic / (ev_avg * 1e-3) / 1e9 / HBM_PEAK_GBS
     if w.dtype != "f32":
         roofline["mfma_frac"] = flops / (ev_avg * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
 

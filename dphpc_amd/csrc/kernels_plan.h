@@ -147,13 +147,19 @@ __global__ __launch_bounds__(256) void k_check_index(const int32_t *__restrict__
 
 // rowptr -> row index per stored entry (what the flat kernels read).  A wavefront
 // takes 64 rows: short rows are written by their own lane, long ones by the
-// whole wavefront.
+// whole wavefront.  Positions outside [0, limit) are never written, whatever the
+// row pointer holds (it may come unvalidated from the caller).
 __global__ __launch_bounds__(256) void k_expand_rows(const int32_t *__restrict__ rowptr, int M,
-                                                     int32_t *__restrict__ rowidx) {
+                                                     int32_t *__restrict__ rowidx, int64_t limit) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = lane_id();
     int32_t s = 0, e = 0;
-    if (i < M) { s = rowptr[i]; e = rowptr[i + 1]; }
+    if (i < M) {
+        s = rowptr[i];
+        e = rowptr[i + 1];
+        s = s < 0 ? 0 : s;
+        e = (int64_t)e > limit ? (int32_t)limit : e;
+    }
     const int len = e - s;
     constexpr int SHORT = 8;
     if (len <= SHORT) {

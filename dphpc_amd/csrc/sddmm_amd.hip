@@ -554,12 +554,26 @@ int classify_rows_items(sddmm_ctx *c, bool with_short_list = true) {
         c->n_short_list = (int64_t)c->pc.nnz_short;
         if ((int64_t)c->raw.short_scanned != c->n_short_list)
             return fail(c, SDDMM_ERR_HIP, "internal: scan of the short rows disagrees with their entry count");
-        if (c->n_short_list > c->short_list_cap) {
+        // The list is a convenience of 8 bytes per entry of a short row.  Above a cap
+        // (SDDMM_SHORT_LIST_MAX entries, default 2^27 = 1 GiB), or when the device cannot
+        // hold it, the launch walks the short rows themselves (short_rows_body) instead.
+        const int64_t cap = (int64_t)env_int("SDDMM_SHORT_LIST_MAX", 1 << 27);
+        if (c->n_short_list > cap) c->use_short_list = false;
+        if (c->use_short_list && c->n_short_list > c->short_list_cap) {
             dfree(c->d_short_list);
             c->short_list_cap = 0;
-            ALLOC_TRY(c, c->d_short_list, (size_t)c->n_short_list * sizeof(int2));
-            c->short_list_cap = c->n_short_list;
+            void *p = nullptr;
+            if (hipMalloc(&p, (size_t)c->n_short_list * sizeof(int2)) == hipSuccess && p) {
+                c->d_short_list = static_cast<decltype(c->d_short_list)>(p);
+                c->short_list_cap = c->n_short_list;
+            } else {
+                (void)hipGetLastError();                       // the failed allocation is not an error of the plan
+                c->use_short_list = false;
+            }
         }
+        if (!c->use_short_list) c->n_short_list = 0;
+    }
+    if (c->use_short_list) {
         SDDMM_LAUNCH(c, k_short_list_write, nb, SCAN_BLOCK, c->d_rowptr,
                            (const unsigned char *)(c->owner_active ? c->d_owner : nullptr), c->sM, c->ts,
                            (const unsigned int *)c->d_short_sums, c->d_short_list);
@@ -958,7 +972,7 @@ int ensure_rowidx(sddmm_ctx *c) {
     c->own_rowidx = true;
     if (c->sM > 0 && c->nnz > 0)
         SDDMM_LAUNCH(c, k_expand_rows, grid_for(c->sM, 256), 256, c->d_rowptr, c->sM,
-                           c->d_rowidx);
+                           c->d_rowidx, c->nnz);
     LAUNCH_CHECK(c);
     return SDDMM_OK;
 }
@@ -1501,10 +1515,13 @@ int sddmm_run(sddmm_ctx *c) {
     return SDDMM_OK;
 }
 
-// items of the fused kernel: the rows of more than FUSED_ROW_MAX entries, cut into segments of SDDMM_SEG entries
+// items of the fused kernel: the rows of more than FUSED_ROW_MAX entries, cut into segments of
+// SDDMM_FUSED_SEG entries (default 2048, shortened below when there are few items; a knob of its own,
+// apart from SDDMM_SEG of the plain SDDMM, because the pieces of a row add to O atomically: the segment
+// length decides which rows are summed in an order that may differ from run to run)
 static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
     if (c->fused_items_valid && c->fused_items_panels == (panel_owner != nullptr)) return SDDMM_OK;
-    int seg = std::max(WAVE, env_int("SDDMM_SEG", 2048));
+    int seg = std::max(WAVE, env_int("SDDMM_FUSED_SEG", 2048));
     const int64_t nb = ((int64_t)c->sM + SCAN_TILE - 1) / SCAN_TILE;
     const int arc = ensure_arena(c);
     if (arc) return arc;
@@ -1535,7 +1552,7 @@ static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
         const PlanCounters first = summarize(tmp);
         const int64_t item_entries = (int64_t)(first.nnz_medium + first.nnz_long);
         // (rows of up to 128 bytes; at 256 bytes it changes nothing, at 1 KiB the adds of 256 floats per piece lose 4 %)
-        if ((int64_t)tmp.n_items > 0 && (int64_t)tmp.n_items < 4096 && !getenv("SDDMM_SEG") &&
+        if ((int64_t)tmp.n_items > 0 && (int64_t)tmp.n_items < 4096 && !getenv("SDDMM_FUSED_SEG") &&
             (size_t)c->K * elem_size(c->dtype) <= 128) {
             int shorter = (int)std::min<int64_t>(seg, ((item_entries / 8192 + WAVE - 1) / WAVE) * WAVE);
             shorter = std::max(shorter, 256);
@@ -1798,7 +1815,8 @@ int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, cons
     c.d_sval = const_cast<float *>(d_sval);
     c.dP = dP;
     c.d_rowidx = rowidx;                       // every position below nnz is rewritten: nothing to clear
-    SDDMM_LAUNCH(&c, k_expand_rows, grid_for(M, 256), 256, c.d_rowptr, M, rowidx);
+    // (bounded by nnz: a row pointer that runs past it cannot make the kernel leave the array)
+    SDDMM_LAUNCH(&c, k_expand_rows, grid_for(M, 256), 256, c.d_rowptr, M, rowidx, nnz);
     launch_flat(&c);
     if (hipGetLastError() != hipSuccess) return SDDMM_ERR_HIP;
     if (c.oversize) return SDDMM_ERR_UNSUPPORTED;

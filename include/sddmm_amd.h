@@ -202,11 +202,17 @@ int sddmm_time_region(sddmm_ctx *ctx, int reps, int include_plan, float *total_m
  *   - dA [M x K], dB [N x K] row-major fp32, 16-byte aligned; d_rowptr[M+1], d_col[nnz],
  *     d_sval[nnz], dP[nnz]; P is complete when `stream` has executed the call;
  *   - the structure is NOT validated here (that needs a read-back): pass arrays that
- *     sddmm_set_csr_device would accept;
+ *     sddmm_set_csr_device would accept; row pointer values beyond nnz are clamped when
+ *     the row indices are written, so a bad row pointer cannot write outside the array;
+ *   - every process that loads the library reserves the array on each device it uses,
+ *     whether or not this entry point is called; a deployment that never calls it can
+ *     build the library with a smaller -DSDDMM_NOALLOC_MAX_NNZ=<n>;
  *   - nnz > SDDMM_NOALLOC_MAX_NNZ returns SDDMM_ERR_TOO_LARGE and launches nothing;
  *   - all calls on one device share the array: calls that may overlap on one GPU
  *     (different streams, different threads) race; order them on one stream. */
+#ifndef SDDMM_NOALLOC_MAX_NNZ
 #define SDDMM_NOALLOC_MAX_NNZ (1 << 24)
+#endif
 int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, const float *dB,
                          const int32_t *d_rowptr, const int32_t *d_col, const float *d_sval, float *dP,
                          void *stream);

@@ -53,7 +53,7 @@ def test_fused_random(engine_factory, K):
 
 def test_fused_rows_split_into_segments(engine_factory, monkeypatch):
     """Rows longer than a segment are accumulated by several wavefronts (atomic adds)."""
-    monkeypatch.setenv("SDDMM_SEG", "128")
+    monkeypatch.setenv("SDDMM_FUSED_SEG", "128")
     rng = np.random.default_rng(31)
     M, N, K = 40, 3000, 32
     rows = [np.sort(rng.choice(N, int(rng.choice([0, 5, 127, 128, 129, 700, 2500])), replace=False)) for _ in range(M)]

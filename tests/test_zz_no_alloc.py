@@ -136,3 +136,92 @@ def test_sizes_beyond_the_static_buffer_and_bad_arguments_are_refused():
         assert L.sddmm_launch_noalloc(10, 10, 8, 5, C.c_void_p(d.value + 4), d, d, d, d, d, None) == capi.ERR_INVALID
     finally:
         hip.free_all()
+
+
+def test_row_pointer_beyond_nnz_writes_nothing_outside_the_output():
+    """A row pointer whose tail runs past the nnz argument (the structure is not validated by
+    this entry point) must not make the library write outside its own array or outside
+    P[0, nnz): the entries below nnz come out as usual, a guard area behind P stays untouched."""
+    L = capi.load_library()
+    hip = Hip()
+    try:
+        w = W.make("mixed_density", "small", K=32)
+        cut = int(w.rowptr[w.M // 2])                  # entries of the first half of the rows
+        assert 0 < cut < w.nnz
+        bad_rowptr = w.rowptr.copy()
+        bad_rowptr[w.M // 2 + 1:] += 1 << 26           # far beyond nnz and beyond the static array
+        bad_rowptr[-1] = np.iinfo(np.int32).max
+        dA, dB = hip.upload(w.A), hip.upload(w.B)
+        d_rp, d_col, d_val = hip.upload(bad_rowptr), hip.upload(w.col), hip.upload(w.sval)
+        guard = 4096
+        sentinel = np.full(cut + guard, -123.25, f32)
+        dP = hip.upload(sentinel)
+        # first a good call, so that every row index the flat kernel may read below is a valid row
+        good = _noalloc(L, hip, w)
+        rc = L.sddmm_launch_noalloc(w.M, w.N, w.K, cut, dA, dB, d_rp, d_col, d_val, dP, None)
+        assert rc == 0, L.sddmm_strerror(rc)
+        got = hip.download(dP, cut + guard, f32)
+        np.testing.assert_array_equal(got[cut:], sentinel[cut:])
+        np.testing.assert_array_equal(got[:cut].view(np.uint32), good[:cut].view(np.uint32))
+    finally:
+        hip.free_all()
+
+
+def test_under_graph_capture_and_without_allocating():
+    """What the entry point is for: after the warm-up call (nnz = 0, outside the capture) one call
+    is captured into a HIP graph -- kernels only -- and the graph launched twice, with eager work
+    in between; both replays give the flat strategy's values.  The free device memory is the same
+    before and after an eager call."""
+    L = capi.load_library()
+    hip = Hip()
+    h = hip.h
+    vp = C.c_void_p
+    h.hipStreamCreate.argtypes = [C.POINTER(vp)]
+    h.hipStreamDestroy.argtypes = [vp]
+    h.hipStreamSynchronize.argtypes = [vp]
+    h.hipStreamBeginCapture.argtypes = [vp, C.c_int]
+    h.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+    h.hipGraphInstantiate.argtypes = [C.POINTER(vp), vp, vp, vp, C.c_size_t]
+    h.hipGraphLaunch.argtypes = [vp, vp]
+    h.hipGraphExecDestroy.argtypes = [vp]
+    h.hipGraphDestroy.argtypes = [vp]
+    h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    h.hipMemsetAsync.argtypes = [vp, C.c_int, C.c_size_t, vp]
+    stream, graph, gexec = vp(), vp(), vp()
+    try:
+        w = W.make("power_law", "small", K=32)
+        want = _flat_through_a_context(w)
+        dA, dB = hip.upload(w.A), hip.upload(w.B)
+        d_rp, d_col, d_val = hip.upload(w.rowptr), hip.upload(w.col), hip.upload(w.sval)
+        dP = hip.zeros(4 * w.nnz)
+        assert h.hipStreamCreate(C.byref(stream)) == 0
+        assert L.sddmm_launch_noalloc(w.M, w.N, w.K, 0, None, None, d_rp, None, None, None, stream) == 0   # warm-up
+        assert L.sddmm_launch_noalloc(w.M, w.N, w.K, w.nnz, dA, dB, d_rp, d_col, d_val, dP, stream) == 0   # code loaded
+        assert h.hipStreamSynchronize(stream) == 0
+        free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        assert h.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+        assert L.sddmm_launch_noalloc(w.M, w.N, w.K, w.nnz, dA, dB, d_rp, d_col, d_val, dP, stream) == 0
+        assert h.hipStreamSynchronize(stream) == 0
+        assert h.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+        assert free0.value == free1.value
+
+        assert h.hipStreamBeginCapture(stream, 0) == 0                       # hipStreamCaptureModeGlobal
+        rc = L.sddmm_launch_noalloc(w.M, w.N, w.K, w.nnz, dA, dB, d_rp, d_col, d_val, dP, stream)
+        assert h.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert rc == 0, L.sddmm_strerror(rc)
+        assert h.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for replay in range(2):
+            assert h.hipMemsetAsync(dP, 0, 4 * w.nnz, stream) == 0           # eager work between the replays
+            assert h.hipStreamSynchronize(stream) == 0
+            assert h.hipGraphLaunch(gexec, stream) == 0
+            assert h.hipStreamSynchronize(stream) == 0
+            got = hip.download(dP, w.nnz, f32)
+            np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32), err_msg="replay %d" % replay)
+    finally:
+        if gexec:
+            h.hipGraphExecDestroy(gexec)
+        if graph:
+            h.hipGraphDestroy(graph)
+        if stream:
+            h.hipStreamDestroy(stream)
+        hip.free_all()
