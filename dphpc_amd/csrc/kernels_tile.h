@@ -1432,9 +1432,28 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
     const int prow = lane >> 3, punit = lane & 7;
     // fp32 rows of 128 bytes and more: 4x4 blocks, every multiply-add useful (see above)
     constexpr bool BLOCKS = DT == DT_F32 && STEPS % 2 == 0;
+    // the 8 rows of a panel have one length and follow each other in the CSR arrays
+    const int rs0 = __builtin_amdgcn_readfirstlane(it.pad);
+    const int row_len = __builtin_amdgcn_readfirstlane(rowptr[row0 + 1]) - rs0;
+    const int64_t out_row = (int64_t)rs0 + (int64_t)prow * row_len;   // this lane's S/P row starts here
+    // ROTATE: the S/P window of a row lags the compute window by `rot` 16-byte units, chosen so
+    // that the 128 bytes which the 8 lanes of a row read and write per pair are one whole line of
+    // the output array (rows start wherever the CSR arrays put them).  A lane takes unit
+    // (punit - rot) mod 8 of every pair; lanes with punit < rot store it one pair later, next to
+    // the first units of that pair (`held` keeps it until then), and one more store-only step
+    // follows the last pair.  Unrotated accesses straddle two lines each: every line of S is then
+    // requested twice and every line of P written in two halves, and both wait in L2 in between.
+    constexpr bool ROTATE = !FUSED;
+    int rot = 0, src_unit = punit;
+    if constexpr (ROTATE) {
+        rot = (int)(((((uintptr_t)P) >> 2) + (uint64_t)(out_row + start)) & 31u) >> 2;
+        src_unit = (punit - rot) & 7;
+    }
+    const bool use_now = punit >= rot;
+    const bool any_rot = ROTATE && __ballot(rot != 0) != 0;
     const int to_memory_from =
-        (BLOCKS ? 32 * (prow >> 2) + 16 * (punit >> 2) + 4 * (punit & 3) + (prow & 3)
-                : 16 * (punit & 3) + prow + 8 * (punit >> 2)) << 2;
+        (BLOCKS ? 32 * (prow >> 2) + 16 * (src_unit >> 2) + 4 * (src_unit & 3) + (prow & 3)
+                : 16 * (src_unit & 3) + prow + 8 * (src_unit >> 2)) << 2;
     constexpr int ROW_UNITS = STEPS * 4;
     // groups of 16 columns in flight; rows of 512 bytes and more leave registers for two
     constexpr int GROUPS = STEPS >= 8 ? 2 : 4;
@@ -1454,10 +1473,6 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) a[s] = src[s * 4];
     }
-    // the 8 rows of a panel have one length and follow each other in the CSR arrays
-    const int rs0 = __builtin_amdgcn_readfirstlane(it.pad);
-    const int row_len = __builtin_amdgcn_readfirstlane(rowptr[row0 + 1]) - rs0;
-    const int64_t out_row = (int64_t)rs0 + (int64_t)prow * row_len;   // this lane's S/P row starts here
     const int last = end - 1;
     auto cols_of_chunk = [&](int base) {                        // column of entry base + lane (clamped)
         const int e = base + lane < last ? base + lane : last;
@@ -1479,7 +1494,9 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         // entries are not all inside the item fetch their S values again.
         o.s = F4u{0.f, 0.f, 0.f, 0.f};
         if ((u & 1) == 0) {
-            const int e = g0 + 4 * punit < row_len - 4 ? g0 + 4 * punit : row_len - 4;
+            int e = g0 + 4 * (punit - rot);
+            e = e < row_len - 4 ? e : row_len - 4;
+            e = e > 0 ? e : 0;
             o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
         }
         return o;
@@ -1574,10 +1591,13 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         }
     };
     // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
+    float held[4] = {0.f, 0.f, 0.f, 0.f};                        // ROTATE: the unit taken from the previous pair
     auto compute_store_pair = [&](const Oper &o0, const Oper &o1, int g0) {
-        if (g0 >= end) return;                                   // wave-uniform
-        float r0, r1, r2, r3;
-        if constexpr (BLOCKS) {
+        if (g0 >= end + (any_rot ? 32 : 0)) return;              // wave-uniform
+        const bool past = g0 >= end;                             // the store-only step after the last pair
+        float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
+        if (past) {
+        } else if constexpr (BLOCKS) {
             f32x4_t lo0, hi0, lo1, hi1;
             compute_blocks(o0, lo0, hi0);
             compute_blocks(o1, lo1, hi1);                        // columns clamped past the end: computed, not stored
@@ -1609,11 +1629,19 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         }
         const uint4 m = permute4(to_memory_from, __builtin_bit_cast(uint32_t, r0), __builtin_bit_cast(uint32_t, r1),
                                  __builtin_bit_cast(uint32_t, r2), __builtin_bit_cast(uint32_t, r3));
-        const float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
-        const float d2 = __builtin_bit_cast(float, m.z), d3 = __builtin_bit_cast(float, m.w);
-        const int e = g0 + 4 * punit;
+        float d0 = __builtin_bit_cast(float, m.x), d1 = __builtin_bit_cast(float, m.y);
+        float d2 = __builtin_bit_cast(float, m.z), d3 = __builtin_bit_cast(float, m.w);
+        if constexpr (ROTATE) {
+            const float n0 = d0, n1 = d1, n2 = d2, n3 = d3;
+            d0 = use_now ? n0 : held[0]; d1 = use_now ? n1 : held[1];
+            d2 = use_now ? n2 : held[2]; d3 = use_now ? n3 : held[3];
+            held[0] = n0; held[1] = n1; held[2] = n2; held[3] = n3;
+        }
+        const int e = g0 + 4 * (punit - rot);
         float p[4] = {0.f, 0.f, 0.f, 0.f};                       // FUSED: the P values, 0 past the end of the item
-        if (e + 4 <= end) {
+        if (e < start) {
+            // ROTATE, first pair: these lanes' first unit comes with the next pair
+        } else if (e + 4 <= end) {
             // four consecutive entries inside the item (so the S window was not clamped)
             F4u out{d0 * o0.s.x, d1 * o0.s.y, d2 * o0.s.z, d3 * o0.s.w};
             *reinterpret_cast<F4u *>(P + out_row + e) = out;
@@ -1658,7 +1686,8 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         o[u] = load_oper(cc0, u, start + 16 * u);
         __builtin_amdgcn_sched_barrier(0);
     }
-    for (int base = start; base < end; base += CHUNK) {
+    const int walk_end = end + (any_rot ? 32 : 0);
+    for (int base = start; base < walk_end; base += CHUNK) {
         const int cc_nn = cols_of_chunk(base + 2 * CHUNK);
 #pragma unroll
         for (int u = 0; u < GROUPS; u += 2) {
