@@ -506,6 +506,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_union_tiles(
 // is GATHERED_BASE + its index, its rows are listed in a table (16 per strip, -1 for
 // a missing row).
 constexpr int GATHERED_BASE = 1 << 30;
+constexpr int TILE_WINDOW = 4;                  // descriptors per window (what a wavefront of the tile kernels takes)
 
 __global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__restrict__ rowptr,
                                                            const int32_t *__restrict__ col, int M,
@@ -537,38 +538,50 @@ __global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__rest
     }
 }
 
-// Rows, extent and column span of gathered strip vs; lanes 0..15 keep one row each.
+// Gathered strips come in PAIRS: 32 consecutive candidates of the sorted order, the first 16
+// as strip 2p, the rest as strip 2p+1, with ONE list of tile columns -- every tile column that
+// any of the 32 rows touches -- so that the two strips have the same descriptors in the same
+// order and a wavefront can use every B tile it loads for both (tile_window_pair_wave).  The
+// list is padded with absent tile columns to a multiple of TILE_WINDOW, so that no window of
+// four descriptors holds two strips, and stored window by window, the four descriptors of
+// strip 2p followed by the four of strip 2p+1.
+//
+// Rows, extent and column span of pair vp; lanes 0..31 keep one row each.
 struct GatheredHead {
     int row, s, e;        // per lane (row -1: none)
     int lo, span;         // wave-uniform, in tile columns
+    int halves;           // wave-uniform: 2 when the second strip has rows, else 1
     int64_t entries;      // wave-uniform
 };
 __device__ __forceinline__ GatheredHead gathered_head(const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const unsigned long long *__restrict__ sorted_keys,
-                                                      int64_t n_cand, int64_t vs) {
+                                                      int64_t n_cand, int64_t vp) {
     GatheredHead h;
     const int lane = lane_id();
-    const int64_t idx = vs * 16 + lane;
-    h.row = lane < 16 && idx < n_cand ? (int)(unsigned int)sorted_keys[idx] : -1;   // low half of the key
+    const int64_t idx = vp * 32 + lane;
+    h.row = lane < 32 && idx < n_cand ? (int)(unsigned int)sorted_keys[idx] : -1;   // low half of the key
     h.s = h.row >= 0 ? rowptr[h.row] : 0;
     h.e = h.row >= 0 ? rowptr[h.row + 1] : 0;
     const bool has = h.e > h.s;
     const int first = has ? (col[h.s] >> 4) : INT32_MAX;
     const int last = has ? (col[h.e - 1] >> 4) : -1;
-    // lanes 16..63 hold the neutral values, so the 16-lane reductions of row 0 are the strip's
-    const int l = __builtin_amdgcn_readfirstlane(min16(first));
-    const int hneg = __builtin_amdgcn_readfirstlane(min16(-last));
+    // lanes 32..63 hold the neutral values; the 16-lane reductions of rows 0 and 1 of the wave make the pair's
+    const int l16 = min16(first), h16 = min16(-last), n16 = sum16(h.e - h.s);
+    const int l0 = __builtin_amdgcn_readlane(l16, 0), l1 = __builtin_amdgcn_readlane(l16, 16);
+    const int g0 = __builtin_amdgcn_readlane(h16, 0), g1 = __builtin_amdgcn_readlane(h16, 16);
+    const int l = l0 < l1 ? l0 : l1, hneg = g0 < g1 ? g0 : g1;
     h.lo = l;
     h.span = l == INT32_MAX ? 0 : -hneg - l + 1;
-    h.entries = (int64_t)__builtin_amdgcn_readfirstlane(sum16(h.e - h.s));
+    h.entries = (int64_t)__builtin_amdgcn_readlane(n16, 0) + (int64_t)__builtin_amdgcn_readlane(n16, 16);
+    h.halves = vp * 32 + 16 < n_cand ? 2 : 1;
     return h;
 }
 
-// One workgroup of 16 wavefronts per gathered strip: wave i streams row i of the
-// strip into the strip's tile-column bitmap in LDS (the rows are not neighbours in
-// the CSR arrays, so they are 16 independent streams).  Returns false when a row is
-// not sorted.  Every wave of the workgroup must call it.
+// One workgroup of 16 wavefronts per pair: wave i streams rows i and 16+i of the pair into the
+// pair's tile-column bitmap in LDS (the rows are not neighbours in the CSR arrays, so they are
+// independent streams).  Returns false when a row is not sorted.  Every wave of the workgroup
+// must call it.
 constexpr int GATHERED_BLOCK = 16 * WAVE;
 
 __device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, const GatheredHead &h, unsigned int *bm,
@@ -578,30 +591,34 @@ __device__ __forceinline__ bool gathered_mark(const int32_t *__restrict__ col, c
     if (threadIdx.x == 0) *unsorted_flag = 0;
     __syncthreads();
     const int wi = wave_in_block();
-    const int si = __builtin_amdgcn_readlane(h.s, wi), ei = __builtin_amdgcn_readlane(h.e, wi);
-    if (ei > si) {                                   // wave-uniform
-        int64_t descents = 0;
-        (void)strip_scan<1>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
-        if (descents != 0 && lane_id() == 0) atomicOr(unsorted_flag, 1);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int si = half ? __builtin_amdgcn_readlane(h.s, (wi & 15) + 16) : __builtin_amdgcn_readlane(h.s, wi & 15);
+        const int ei = half ? __builtin_amdgcn_readlane(h.e, (wi & 15) + 16) : __builtin_amdgcn_readlane(h.e, wi & 15);
+        if (ei > si) {                               // wave-uniform
+            int64_t descents = 0;
+            (void)strip_scan<1>(col, si, ei, INT64_MAX, h.lo, h.span, bm, &descents);
+            if (descents != 0 && lane_id() == 0) atomicOr(unsorted_flag, 1);
+        }
     }
     __syncthreads();
     return *unsorted_flag == 0;
 }
 
-// pass 1 of the gathered strips: tiles per strip (0: not taken), the strip's row
-// table, ownership of the rows of a taken strip.
+// pass 1 of the gathered strips: descriptors per strip of the pair (0: not taken; the same for
+// both strips), the strips' row table, ownership of the rows of a taken pair.
 __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_count(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
     const unsigned long long *__restrict__ sorted_keys,
-    int64_t n_cand, int64_t n_vstrips, int min_fill, unsigned int *__restrict__ vstrip_ntiles,
+    int64_t n_cand, int64_t n_vpairs, int min_fill, unsigned int *__restrict__ vstrip_ntiles,
     int32_t *__restrict__ vrows, unsigned char *__restrict__ owner, DevCounters *pc) {
     __shared__ unsigned int bm[STRIP_BM_WORDS];
     __shared__ int unsorted_flag, tile_total;
-    const int64_t vs = blockIdx.x;
+    const int64_t vp = blockIdx.x;
     const int lane = lane_id();
     const bool first = wave_in_block() == 0;
-    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);   // the same in every wave
-    if (first && lane < 16) vrows[vs * 16 + lane] = h.row;
+    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vp);   // the same in every wave
+    if (first && lane < 32) vrows[vp * 32 + lane] = h.row;
     int tiles = 0;
     bool take = false;
     if (h.span > 0 && h.span <= STRIP_BM_WORDS * 32 && h.entries >= min_fill) {   // workgroup-uniform
@@ -615,36 +632,65 @@ __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_count(
         if (lane == 0 && t) atomicAdd(&tile_total, t);
         __syncthreads();
         tiles = tile_total;
-        take = sorted && tiles > 0 && h.entries >= (int64_t)min_fill * tiles;
+        // the threshold is per 16x16 tile: each tile column of the pair is one tile per strip that has rows
+        take = sorted && tiles > 0 && h.entries >= (int64_t)min_fill * tiles * h.halves;
     }
+    const int padded = (tiles + TILE_WINDOW - 1) / TILE_WINDOW * TILE_WINDOW;
     if (first) {
         if (take && h.row >= 0) owner[h.row] = 3;
         if (lane == 0) {
-            vstrip_ntiles[vs] = take ? (unsigned int)tiles : 0u;
+            vstrip_ntiles[2 * vp] = take ? (unsigned int)padded : 0u;
+            vstrip_ntiles[2 * vp + 1] = take ? (unsigned int)padded : 0u;
             if (take) {
-                spread_add(pc, K_TILES, (unsigned long long)tiles);
+                spread_add(pc, K_TILES, 2ull * (unsigned long long)padded);
                 spread_add(pc, K_NNZ_TILES, (unsigned long long)h.entries);
             }
         }
     }
 }
 
-// pass 2 of the gathered strips: strip and tile column of every descriptor
+// A descriptor that stands for nothing (no row has an entry in it): complete, k_tile_rows skips it.
+__device__ __forceinline__ void write_empty_desc(TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols,
+                                                 int64_t at, int strip, int tj) {
+    int4 *d = reinterpret_cast<int4 *>(tiles + at);
+    d[0] = make_int4(strip, tj, 1, 0);
+#pragma unroll
+    for (int k = 1; k < (int)(sizeof(TileDesc) / 16); ++k) d[k] = make_int4(0, 0, 0, 0);
+    write_aligned_cols(tile_cols, at, tj);
+}
+
+// pass 2 of the gathered strips: strip and tile column of every descriptor, window by window
+// (descriptor 8k + 4h + j of the pair: strip h, the (4k+j)-th tile column).  `tiles` / `tile_cols`
+// point at the first gathered descriptor; the `lead` descriptors before it (fewer than
+// TILE_WINDOW) fill the last window of the strips that precede the gathered ones.
 __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
     const int32_t *__restrict__ rowptr, const int32_t *__restrict__ col,
     const unsigned long long *__restrict__ sorted_keys,
-    int64_t n_cand, int64_t n_vstrips, const unsigned int *__restrict__ vstrip_ntiles,
-    const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols) {
+    int64_t n_cand, int64_t n_vpairs, const unsigned int *__restrict__ vstrip_ntiles,
+    const unsigned int *__restrict__ vstrip_off, TileDesc *__restrict__ tiles, int32_t *__restrict__ tile_cols,
+    int lead) {
     __shared__ unsigned int bm[STRIP_BM_WORDS];
     __shared__ int unsorted_flag;
-    const int64_t vs = blockIdx.x;
-    if (vstrip_ntiles[vs] == 0) return;              // workgroup-uniform
+    const int64_t vp = blockIdx.x;
+    // (strip -1 is nobody's: the window that holds them is walked tile by tile, and they write nothing)
+    if (vp == 0 && (int)threadIdx.x < lead) write_empty_desc(tiles, tile_cols, -(int64_t)lead + threadIdx.x, -1, 0);
+    const unsigned int per_strip = vstrip_ntiles[2 * vp];
+    if (per_strip == 0) return;                      // workgroup-uniform
     const int lane = lane_id();
-    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vs);
+    const GatheredHead h = gathered_head(rowptr, col, sorted_keys, n_cand, vp);
     (void)gathered_mark(col, h, bm, &unsorted_flag);
     if (wave_in_block() != 0) return;                // the first wave writes the descriptors in column order
     const int words = (h.span + 31) >> 5;
-    int64_t run = vstrip_off[vs];
+    const int64_t base = vstrip_off[2 * vp];
+    const int strip0 = GATHERED_BASE + (int)(2 * vp);
+    auto put = [&](int rank, int tj) {
+        const int64_t at = base + 2 * TILE_WINDOW * (rank / TILE_WINDOW) + (rank % TILE_WINDOW);
+        *reinterpret_cast<int4 *>(tiles + at) = make_int4(strip0, tj, 0, 0);
+        write_aligned_cols(tile_cols, at, tj);
+        *reinterpret_cast<int4 *>(tiles + at + TILE_WINDOW) = make_int4(strip0 + 1, tj, 0, 0);
+        write_aligned_cols(tile_cols, at + TILE_WINDOW, tj);
+    };
+    int run = 0, top = -1;
     for (int wb = 0; wb < words; wb += WAVE) {
         const int w = wb + lane;
         unsigned int x = w < words ? bm[w] : 0u;
@@ -654,16 +700,25 @@ __global__ __launch_bounds__(GATHERED_BLOCK) void k_gathered_tiles(
             const int up = __shfl_up(incl, o, WAVE);
             if (lane >= o) incl += up;
         }
-        int64_t at = run + (incl - n);
+        int rank = run + (incl - n);
         while (x) {
             const int b = __builtin_ctz(x);
             x &= x - 1;
-            *reinterpret_cast<int4 *>(tiles + at) = make_int4(GATHERED_BASE + (int)vs, h.lo + w * 32 + b, 0, 0);
-            write_aligned_cols(tile_cols, at, h.lo + w * 32 + b);
-            ++at;
+            const int tj = h.lo + w * 32 + b;
+            put(rank, tj);
+            top = tj;                                 // ascending inside a lane and from lane to lane
+            ++rank;
         }
         run += __builtin_amdgcn_readlane(incl, WAVE - 1);
     }
+    // the padding: tile columns beyond the pair's last one, which no row of the pair has
+    for (int o = WAVE / 2; o > 0; o >>= 1) {
+        const int other = __shfl_xor(top, o, WAVE);
+        top = other > top ? other : top;
+    }
+    // (k_tile_rows gives them their per-row positions like any other descriptor: the masks come out
+    // empty, the positions say where a row's entries before that column end)
+    if (run + lane < (int)per_strip) put(run + lane, top + 1 + lane);
 }
 
 // pass 3: one thread per (descriptor, row): CSR position of the row's first entry
@@ -912,7 +967,6 @@ __device__ __forceinline__ void tile_wave(const void *__restrict__ A, const void
 //
 // A window whose descriptors are not plain aligned tiles of one strip (a strip ends
 // inside it, union tiles) is flagged by the plan and walked tile by tile (tile_wave).
-constexpr int TILE_WINDOW = 4;
 constexpr int WIN_PITCH = 20;                 // floats per result column in LDS: 16 rows, padded, 16-byte aligned
 constexpr int WIN_LDS_FLOATS = TILE_WINDOW * 16 * WIN_PITCH;
 
@@ -923,14 +977,15 @@ struct alignas(16) TileWindow {               // lane l < 48 loads dword l
     int32_t tj[TILE_WINDOW];   // tile columns, -1 where the window has fewer tiles
     int32_t flags;       // != 0: walk the window tile by tile
     int32_t maxcnt;      // largest cnt
-    int32_t pad[2];
+    int32_t paired;      // != 0: a window of a pair of gathered strips (same tile columns as its neighbour)
+    int32_t pad;
 };
 static_assert(sizeof(TileWindow) == 192, "TileWindow layout");
 
 // plan: one thread per (window, strip row)
 __global__ __launch_bounds__(256) void k_tile_windows(const int32_t *__restrict__ vrows, int M, int64_t nnz,
                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
-                                                      int64_t union_lo, int64_t union_hi,
+                                                      int64_t union_lo, int64_t union_hi, int64_t gathered_lo,
                                                       TileWindow *__restrict__ win, int64_t n_win) {
     const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t w = slot >> 4;
@@ -969,7 +1024,8 @@ __global__ __launch_bounds__(256) void k_tile_windows(const int32_t *__restrict_
         for (int k = 0; k < TILE_WINDOW; ++k) o->tj[k] = tj[k];
         o->flags = mixed ? 1 : 0;
         o->maxcnt = mx;
-        o->pad[0] = o->pad[1] = 0;
+        o->paired = t0 >= gathered_lo ? 1 : 0;
+        o->pad = 0;
     }
 }
 
@@ -1129,6 +1185,203 @@ __device__ __forceinline__ void tile_window_wave(const void *__restrict__ A, con
     wave_lds_order();                                     // the next window of this wave reuses the buffer
 }
 
+constexpr int PAIR_MAX_STEPS = 4;             // row bytes / 64 up to which pairs of windows share a wavefront
+// Windows wa and wa+1 of a pair of gathered strips on the calling wavefront: the same four tile
+// columns for 2 x 16 rows.  Every B tile is loaded and moved into operand layout once and
+// multiplied with both A panels; the products of the second strip wait in registers while the
+// entries of the first are picked out of the LDS buffer (one buffer, as for a single window).
+template <int DT, int STEPS>
+__device__ __forceinline__ void tile_window_pair_wave(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                                      const int32_t *__restrict__ vrows,
+                                                      const int32_t *__restrict__ tile_cols,
+                                                      const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                      const TileWindow *__restrict__ win, int64_t n_win,
+                                                      const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                                      float *__restrict__ P, int64_t nnz, int64_t wa, float *lds) {
+    if (wa >= n_win) return;
+    const int lane = lane_id();
+    const int li = lane < 48 ? lane : 47;
+    const int dw0 = reinterpret_cast<const int32_t *>(win + wa)[li];
+    const int dw1 = reinterpret_cast<const int32_t *>(win + (wa + 1 < n_win ? wa + 1 : wa))[li];
+    bool plain = wa + 1 < n_win && __builtin_amdgcn_readlane(dw0, 44) == 0 && __builtin_amdgcn_readlane(dw1, 44) == 0 &&
+                 __builtin_amdgcn_readlane(dw0, 46) != 0 && __builtin_amdgcn_readlane(dw1, 46) != 0;
+    int tj[TILE_WINDOW];
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) {
+        tj[k] = __builtin_amdgcn_readlane(dw0, 40 + k);
+        plain = plain && tj[k] == __builtin_amdgcn_readlane(dw1, 40 + k);
+    }
+    if (!plain) {                                         // wave-uniform: one window after the other
+        for (int64_t w = wa; w < wa + 2; ++w)
+            tile_window_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz, w, lds);
+        return;
+    }
+    const int maxcnt0 = __builtin_amdgcn_readlane(dw0, 45), maxcnt1 = __builtin_amdgcn_readlane(dw1, 45);
+    if (maxcnt0 <= 0 && maxcnt1 <= 0) return;
+    const int r16 = lane & 15, q = lane >> 4;        // operand / result layout
+    const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: four neighbouring lanes on 64 bytes of a row
+    const int to_operand_from = (4 * r16 + q) << 2;
+    constexpr uint32_t ROW_UNITS = STEPS * 4;
+    const uint4 *__restrict__ Au = (const uint4 *)A;
+    const uint4 *__restrict__ Bu = (const uint4 *)B;
+    auto to_operand = [&](const uint4 &v) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.w);
+        return r;
+    };
+    // S/P accesses of this lane in either strip: strip row lane>>2, its entries 4(lane&3)+16m.. of the window
+    struct Rows { int p0, cnt; };
+    auto rows_of = [&](int dw) {
+        Rows r;
+        r.p0 = __shfl(dw, 16 + lrow, WAVE);
+        const int cw = __shfl(dw, 32 + (lrow >> 1), WAVE);
+        r.cnt = (lrow & 1) ? (int)((unsigned int)cw >> 16) : (cw & 0xFFFF);
+        return r;
+    };
+    const Rows rows0 = rows_of(dw0), rows1 = rows_of(dw1);
+    auto entry_pos = [&](const Rows &r, int m) {
+        int ws = 4 * lunit + 16 * m;
+        ws = ws < r.cnt - 4 ? ws : r.cnt - 4;
+        ws = ws < 0 ? 0 : ws;
+        const int64_t pos = (int64_t)r.p0 + ws;
+        return pos < nnz - 4 ? pos : nnz - 4;
+    };
+    // ---- second round trip: both A panels, the B tiles, the first column indices and S values ----
+    uint4 a0[STEPS], a1[STEPS];
+    {
+        const int64_t ar0 = __shfl(dw0, lrow, WAVE), ar1 = __shfl(dw1, lrow, WAVE);
+        const uint4 *s0 = Au + ar0 * ROW_UNITS + lunit, *s1 = Au + ar1 * ROW_UNITS + lunit;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) { a0[s] = s0[s * 4]; a1[s] = s1[s * 4]; }
+    }
+    auto load_b = [&](int k, uint4 (&dst)[STEPS]) {
+        int64_t brow = (int64_t)(tj[k] < 0 ? 0 : tj[k]) * 16 + lrow;
+        brow = brow < N ? brow : N - 1;                   // columns past N are in no row's entries
+        const uint4 *src = Bu + brow * ROW_UNITS + lunit;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) dst[s] = src[s * 4];
+    };
+    uint4 b[2][STEPS];                                    // two B tiles in flight
+    load_b(0, b[0]);
+    if (tj[1] >= 0) load_b(1, b[1]);                      // wave-uniform
+    struct Pre { I4u c[2]; F4u s[2]; };
+    auto prefetch = [&](const Rows &r, int iters) {
+        Pre p;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int64_t pos = entry_pos(r, m < iters ? m : 0);
+            p.c[m] = *reinterpret_cast<const I4u *>(col + pos);
+            p.s[m] = *reinterpret_cast<const F4u *>(sval + pos);
+        }
+        return p;
+    };
+    const int iters0 = (maxcnt0 + 15) >> 4, iters1 = (maxcnt1 + 15) >> 4;      // wave-uniform, 0..4
+    const Pre pre0 = prefetch(rows0, iters0);
+    // ---- products: strip 0's into LDS, strip 1's kept ----------------------------------------------
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) { a0[s] = to_operand(a0[s]); a1[s] = to_operand(a1[s]); }
+    f32x4_t keep[TILE_WINDOW];
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) {
+        keep[k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (tj[k] < 0) continue;                          // wave-uniform
+        f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const uint4 bo = to_operand(b[k & 1][s]);
+            if constexpr (DT == DT_BF16) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a0[s]),
+                                                               __builtin_bit_cast(bf16x8_t, bo), acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a1[s]),
+                                                               __builtin_bit_cast(bf16x8_t, bo), acc1, 0, 0, 0);
+            } else if constexpr (DT == DT_F16) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a0[s]),
+                                                              __builtin_bit_cast(half8_t, bo), acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a1[s]),
+                                                              __builtin_bit_cast(half8_t, bo), acc1, 0, 0, 0);
+            } else {
+                const float bf[4] = {__builtin_bit_cast(float, bo.x), __builtin_bit_cast(float, bo.y),
+                                     __builtin_bit_cast(float, bo.z), __builtin_bit_cast(float, bo.w)};
+                const float f0[4] = {__builtin_bit_cast(float, a0[s].x), __builtin_bit_cast(float, a0[s].y),
+                                     __builtin_bit_cast(float, a0[s].z), __builtin_bit_cast(float, a0[s].w)};
+                const float f1[4] = {__builtin_bit_cast(float, a1[s].x), __builtin_bit_cast(float, a1[s].y),
+                                     __builtin_bit_cast(float, a1[s].z), __builtin_bit_cast(float, a1[s].w)};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(f0[i], bf[i], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(f1[i], bf[i], acc1, 0, 0, 0);
+                }
+            }
+        }
+        // the registers of this B tile are free: the tile after the next one
+        if (k + 2 < TILE_WINDOW && tj[k + 2 < TILE_WINDOW ? k + 2 : k] >= 0) load_b(k + 2, b[k & 1]);
+        // result register i of lane (r16, q) is row 4q+i, column r16 of tile k
+        *reinterpret_cast<f32x4_t *>(lds + (k * 16 + r16) * WIN_PITCH + 4 * q) = acc0;
+        keep[k] = acc1;
+    }
+    wave_lds_order();
+    const Pre pre1 = prefetch(rows1, iters1);             // lands while strip 0's entries are written
+    // ---- entries: four per lane, 16 per row and iteration ---------------------------------------------
+    const int t1 = tj[1], t2 = tj[2], t3 = tj[3];
+    auto pick = [&](int c) {
+        const int tc = c >> 4;
+        const int k = (tc == t1 ? 1 : 0) + (tc == t2 ? 2 : 0) + (tc == t3 ? 3 : 0);
+        return lds[(k * 16 + (c & 15)) * WIN_PITCH + lrow];
+    };
+    auto entries = [&](const Rows &r, const Pre &pre, int iters) {
+        for (int m = 0; m < iters; ++m) {
+            I4u c4;
+            F4u s4;
+            if (m < 2) { c4 = pre.c[m]; s4 = pre.s[m]; }
+            else {
+                const int64_t pos = entry_pos(r, m);
+                c4 = *reinterpret_cast<const I4u *>(col + pos);
+                s4 = *reinterpret_cast<const F4u *>(sval + pos);
+            }
+            const bool active = r.cnt >= 4 && 4 * lunit + 16 * m < r.cnt;
+            const F4u out{pick(c4.x) * s4.x, pick(c4.y) * s4.y, pick(c4.z) * s4.z, pick(c4.w) * s4.w};
+            if (active) *reinterpret_cast<F4u *>(P + entry_pos(r, m)) = out;
+        }
+        // rows with one to three entries in the window: entry by entry
+        if (r.cnt > 0 && r.cnt < 4 && lunit == 0) {
+            for (int e = 0; e < r.cnt; ++e) P[(int64_t)r.p0 + e] = pick(col[(int64_t)r.p0 + e]) * sval[(int64_t)r.p0 + e];
+        }
+    };
+    entries(rows0, pre0, iters0);
+    wave_lds_order();
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k)
+        if (tj[k] >= 0) *reinterpret_cast<f32x4_t *>(lds + (k * 16 + r16) * WIN_PITCH + 4 * q) = keep[k];
+    wave_lds_order();
+    entries(rows1, pre1, iters1);
+    wave_lds_order();                                     // the next window of this wave reuses the buffer
+}
+
+// Wavefront `unit` of a tile launch: windows [0, n_single) one per wavefront, the windows after them (pairs of
+// gathered strips) two per wavefront.
+template <int DT, int STEPS>
+__device__ __forceinline__ void tile_unit_wave(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                               const int32_t *__restrict__ vrows, const int32_t *__restrict__ tile_cols,
+                                               const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                               const TileWindow *__restrict__ win, int64_t n_win, int64_t n_single,
+                                               const int32_t *__restrict__ col, const float *__restrict__ sval,
+                                               float *__restrict__ P, int64_t nnz, int64_t unit, float *lds,
+                                               const int32_t *__restrict__ order) {
+    // (rows beyond 256 bytes: the second A panel and the kept products do not fit the registers, the
+    // plan gives such launches one wavefront per window throughout)
+    if (STEPS > PAIR_MAX_STEPS || win == nullptr || unit < n_single) {     // wave-uniform
+        tile_window_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz, unit, lds,
+                                    order);
+        return;
+    }
+    if constexpr (STEPS <= PAIR_MAX_STEPS)
+        tile_window_pair_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
+                                         n_single + 2 * (unit - n_single), lds);
+}
+
 template <int DT, int STEPS>
 __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
                                                 const int32_t *__restrict__ vrows,
@@ -1137,12 +1390,12 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
                                                 const TileWindow *__restrict__ win, int64_t n_win,
                                                 const int32_t *__restrict__ col, const float *__restrict__ sval,
                                                 float *__restrict__ P, int64_t nnz, int64_t nblocks,
-                                                const int32_t *__restrict__ order) {
+                                                const int32_t *__restrict__ order, int64_t n_single) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
-    tile_window_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
-                                blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()], order);
+    tile_unit_wave<DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, n_single, col, sval, P, nnz,
+                              blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()], order);
 }
 
 // Order of the windows for operands that exceed an XCD's L2.  The launch gives every XCD a
@@ -1196,10 +1449,10 @@ __global__ __launch_bounds__(256) void k_window_scatter(const TileDesc *__restri
 // the other; two short launches leave the chip half idle twice, one launch does not.
 // L must be the full-K, 32-bit-offset layout of a row of STEPS * 64 bytes.
 #ifndef SDDMM_FUSED_WAVES
-#define SDDMM_FUSED_WAVES 6
+#define SDDMM_FUSED_WAVES 5
 #endif
 template <class L, int STEPS>
-__global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : STEPS == 4 ? 5 : 1) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
+__global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : STEPS == 4 ? 4 : 1) void k_auto_tiles(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                       const int32_t *__restrict__ rowptr,
                                                       const unsigned char *__restrict__ owner,
                                                       const int32_t *__restrict__ col,
@@ -1212,7 +1465,8 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : STEPS == 4 
                                                       const TileWindow *__restrict__ win, int64_t n_win, int64_t nnz,
                                                       int64_t tile_blocks, int64_t nblocks,
                                                       const int2 *__restrict__ short_list, int64_t n_short_list,
-                                                      int longest_first, const int32_t *__restrict__ order) {
+                                                      int longest_first, const int32_t *__restrict__ order,
+                                                      int64_t n_single) {
     __shared__ __attribute__((aligned(16))) float win_lds[WAVES_PER_BLOCK][WIN_LDS_FLOATS];
     int64_t tile_block = -1, item_block = -1, short_block = -1;
     if (longest_first) {
@@ -1244,9 +1498,9 @@ __global__ __launch_bounds__(BLOCK, STEPS <= 2 ? SDDMM_FUSED_WAVES : STEPS == 4 
         }
     }
     if (tile_block >= 0) {
-        tile_window_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, col, sval, P, nnz,
-                                          tile_block * WAVES_PER_BLOCK + wave_in_block(),
-                                          win_lds[wave_in_block()], order);
+        tile_unit_wave<L::U::DT, STEPS>(A, B, M, N, vrows, tile_cols, tiles, n_tiles, win, n_win, n_single, col, sval, P,
+                                        nnz, tile_block * WAVES_PER_BLOCK + wave_in_block(),
+                                        win_lds[wave_in_block()], order);
         return;
     }
     if (item_block >= 0) {

@@ -83,6 +83,9 @@ struct sddmm_ctx {
     int64_t n_windows = 0, windows_cap = 0;
     bool use_windows = false;        // tile kernels take windows as batches (else they walk them tile by tile)
     int64_t n_tiles_natural = 0;     // descriptors: 16-row strips first, then union strips, then gathered strips
+    int64_t n_tiles_lead = 0;        // empty descriptors that fill the last window before the gathered strips
+    int64_t n_win_single = 0;        // windows taken one per wavefront; the rest (gathered pairs) two per wavefront
+    int64_t n_tile_units = 0;        // wavefronts of a tile launch
     int64_t n_tiles_union = 0, nnz_tiles_union = 0;
     unsigned int *d_ustrip_ntiles = nullptr, *d_ustrip_off = nullptr;
     int64_t ustrips_cap = 0;
@@ -215,8 +218,9 @@ int ensure_arena(sddmm_ctx *c) {
     const size_t o_owner = take((size_t)M + 64);
     const size_t o_strip_n = take((size_t)n_strips * 4), o_strip_o = take((size_t)n_strips * 4);
     const size_t o_ustrip_n = take((size_t)n_strips * 4), o_ustrip_o = take((size_t)n_strips * 4);
-    const size_t o_vstrip_n = take((size_t)n_strips * 4), o_vstrip_o = take((size_t)n_strips * 4);
-    const size_t o_vrows = take((size_t)n_strips * 16 * 4);
+    // (gathered strips come in pairs: up to two more than M / 16)
+    const size_t o_vstrip_n = take((size_t)(n_strips + 2) * 4), o_vstrip_o = take((size_t)(n_strips + 2) * 4);
+    const size_t o_vrows = take((size_t)(n_strips + 2) * 16 * 4);
     const size_t o_panel_n = take((size_t)n_panels * 4), o_panel_o = take((size_t)n_panels * 4);
     const size_t o_keys = take((size_t)(M + 1) * 8), o_sorted = take((size_t)(M + 1) * 8);
     const size_t o_sums = take((size_t)n_sums * 4), o_short_sums = take((size_t)n_sums * 4);
@@ -232,7 +236,8 @@ int ensure_arena(sddmm_ctx *c) {
     c->d_block_sums = (unsigned int *)(b + o_sums);
     c->d_short_sums = (unsigned int *)(b + o_short_sums);
     c->owner_cap = M + 64;
-    c->strips_cap = c->ustrips_cap = c->vstrips_cap = n_strips;
+    c->strips_cap = c->ustrips_cap = n_strips;
+    c->vstrips_cap = n_strips + 2;
     c->panels_cap = n_panels;
     c->cand_cap = M + 1;
     c->block_sums_cap = n_sums;
@@ -458,7 +463,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
     const int64_t waves = short_row_waves(c);
     const int64_t short_blocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t item_blocks = (c->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-    const int64_t tile_blocks = (c->n_windows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t tile_blocks = (c->n_tile_units + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     const int64_t nblocks = short_blocks + item_blocks + tile_blocks;
     // Order of the blocks on every XCD.  Rows of up to 256 bytes: the tile windows (the wavefronts that
     // live longest) start first, then the items, then the chunks of the entry list -- measured
@@ -482,7 +487,7 @@ bool launch_auto_with_tiles(sddmm_ctx *c) {
                                (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows, c->nnz,
                                tile_blocks, nblocks, (const int2 *)(c->use_short_list ? c->d_short_list : nullptr),
                                c->n_short_list, longest_first,
-                               (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr));
+                               (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr), c->n_win_single);
             launched = true;
         }
     });
@@ -611,6 +616,7 @@ int begin_ownership(sddmm_ctx *c) {
     c->owner_active = true;
     c->tiles_active = false;
     c->n_tiles = c->nnz_tiles = c->n_tiles_natural = c->n_tiles_union = c->nnz_tiles_union = 0;
+    c->n_tiles_lead = c->n_win_single = c->n_tile_units = 0;
     c->n_cand = c->n_vstrips = 0;
     c->union_counted = false;
     c->n_panel_items = c->n_panels = c->nnz_panels = 0;
@@ -704,10 +710,12 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill, bool *launched) {
     }
     HIP_TRY(c, rocprim::radix_sort_keys(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
                                         c->stream));
-    c->n_vstrips = (c->n_cand + 15) / 16;
+    // pairs of strips: 32 consecutive candidates share one list of tile columns
+    const int64_t n_vpairs = (c->n_cand + 31) / 32;
+    c->n_vstrips = 2 * n_vpairs;
     ARENA_HOLDS(c, c->n_vstrips, c->vstrips_cap, "gathered strips");
-    SDDMM_LAUNCH(c, k_gathered_count, c->n_vstrips, GATHERED_BLOCK, c->d_rowptr, c->d_col,
-                       (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, min_fill, c->d_vstrip_ntiles,
+    SDDMM_LAUNCH(c, k_gathered_count, n_vpairs, GATHERED_BLOCK, c->d_rowptr, c->d_col,
+                       (const unsigned long long *)c->d_sorted_keys, c->n_cand, n_vpairs, min_fill, c->d_vstrip_ntiles,
                        c->d_vrows, c->d_owner, c->d_pc);
     LAUNCH_CHECK(c);
     rc = device_scan(c, c->d_vstrip_ntiles, c->d_vstrip_off, c->n_vstrips, &c->d_pc->tiles_scanned);
@@ -717,10 +725,15 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill, bool *launched) {
 }
 // after the counters came back
 int plan_gathered_take(sddmm_ctx *c) {
-    c->n_tiles = (int64_t)c->pc.n_tiles + c->n_tiles_union;
-    c->nnz_tiles = (int64_t)c->pc.nnz_tiles + c->nnz_tiles_union;
-    if ((int64_t)c->pc.tiles_scanned != (int64_t)c->pc.n_tiles - c->n_tiles_natural)
+    const int64_t gathered = (int64_t)c->pc.n_tiles - c->n_tiles_natural;
+    if ((int64_t)c->pc.tiles_scanned != gathered)
         return fail(c, SDDMM_ERR_HIP, "internal: gathered tile scan disagrees with tile count");
+    // the gathered descriptors start a window of their own: the strips before them are padded
+    // to a multiple of TILE_WINDOW with descriptors that stand for nothing
+    const int64_t before = c->n_tiles_natural + c->n_tiles_union;
+    c->n_tiles_lead = gathered > 0 ? (TILE_WINDOW - before % TILE_WINDOW) % TILE_WINDOW : 0;
+    c->n_tiles = before + c->n_tiles_lead + gathered;
+    c->nnz_tiles = (int64_t)c->pc.nnz_tiles + c->nnz_tiles_union;
     return SDDMM_OK;
 }
 
@@ -794,11 +807,12 @@ int plan_tiles_fill(sddmm_ctx *c) {
                            c->d_tiles + c->n_tiles_natural, c->d_tile_cols + c->n_tiles_natural * 16);
         LAUNCH_CHECK(c);
     }
-    if (c->n_tiles > c->n_tiles_natural + c->n_tiles_union) {
-        SDDMM_LAUNCH(c, k_gathered_tiles, c->n_vstrips, GATHERED_BLOCK, c->d_rowptr,
-                           c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips, c->d_vstrip_ntiles,
-                           c->d_vstrip_off, c->d_tiles + c->n_tiles_natural + c->n_tiles_union,
-                           c->d_tile_cols + (c->n_tiles_natural + c->n_tiles_union) * 16);
+    const int64_t gathered_lo = c->n_tiles_natural + c->n_tiles_union + c->n_tiles_lead;
+    if (c->n_tiles > gathered_lo) {
+        SDDMM_LAUNCH(c, k_gathered_tiles, c->n_vstrips / 2, GATHERED_BLOCK, c->d_rowptr,
+                           c->d_col, (const unsigned long long *)c->d_sorted_keys, c->n_cand, c->n_vstrips / 2,
+                           c->d_vstrip_ntiles, c->d_vstrip_off, c->d_tiles + gathered_lo,
+                           c->d_tile_cols + gathered_lo * 16, (int)c->n_tiles_lead);
         LAUNCH_CHECK(c);
     }
     SDDMM_LAUNCH(c, k_tile_rows, ((c->n_tiles * 16 + 255) / 256), 256,
@@ -815,6 +829,13 @@ int plan_tiles_fill(sddmm_ctx *c) {
         if (rc) return rc;
     }
     c->use_windows = c->nnz_tiles < (int64_t)env_int("SDDMM_WINDOW_FILL", 176) * c->n_tiles;
+    // wavefronts of a tile launch: one per window, and one per two windows of a pair of gathered strips
+    // (their descriptors come last and fill whole windows, an even number of them)
+    c->n_win_single = c->n_windows;
+    // (rows of up to 256 bytes: beyond that the second A panel and the kept products do not fit the registers)
+    if (c->use_windows && c->n_tiles > gathered_lo && c->tile_steps <= PAIR_MAX_STEPS && env_int("SDDMM_PAIRS", 1) != 0)
+        c->n_win_single = gathered_lo / TILE_WINDOW;
+    c->n_tile_units = c->n_win_single + (c->n_windows - c->n_win_single + 1) / 2;
     if (!c->use_windows) {
         c->tiles_active = true;
         return SDDMM_OK;
@@ -827,7 +848,8 @@ int plan_tiles_fill(sddmm_ctx *c) {
     }
     SDDMM_LAUNCH(c, k_tile_windows, ((c->n_windows * 16 + 255) / 256), 256, (const int32_t *)c->d_vrows, c->sM,
                        c->nnz, (const TileDesc *)c->d_tiles, c->n_tiles, c->n_tiles_natural,
-                       c->n_tiles_natural + c->n_tiles_union, c->d_windows, c->n_windows);
+                       c->n_tiles_natural + c->n_tiles_union, c->n_tiles > gathered_lo ? gathered_lo : c->n_tiles,
+                       c->d_windows, c->n_windows);
     LAUNCH_CHECK(c);
     c->tiles_active = true;
     return SDDMM_OK;
@@ -942,13 +964,13 @@ void launch_panels(sddmm_ctx *c) {
 
 template <int DT, int STEPS>
 void launch_tile_t(sddmm_ctx *c) {
-    const int64_t nblocks = (c->n_windows + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+    const int64_t nblocks = (c->n_tile_units + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     SDDMM_LAUNCH(c, (k_tile<DT, STEPS>), xcd_grid(nblocks), BLOCK,
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
                        (const int32_t *)c->d_tile_cols, (const TileDesc *)c->d_tiles, c->n_tiles,
                        (const TileWindow *)(c->use_windows ? c->d_windows : nullptr), c->n_windows,
                        (const int32_t *)c->d_col, (const float *)c->d_sval, c->dP, c->nnz, nblocks,
-                       (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr));
+                       (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr), c->n_win_single);
 }
 template <int DT>
 void launch_tile_steps(sddmm_ctx *c) {
@@ -1120,7 +1142,9 @@ int do_plan(sddmm_ctx *c, int strategy) {
             if (rc) return rc;
             if (gathered) {
                 bool launched = false;
-                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill)), &launched);
+                // (gathered strips come in pairs that share every B tile they load: a tile pays for
+                // itself at three quarters of the entries a tile of a lone strip needs)
+                rc = plan_gathered_count(c, std::max(1, env_int("SDDMM_GATHERED_FILL", tile_fill * 3 / 4)), &launched);
                 if (rc) return rc;
                 if (launched) {
                     // gathered strips may have taken rows: classify again, one more read-back

@@ -820,6 +820,65 @@ def test_gathered_strips(engine_factory, monkeypatch, K, dtype):
     assert_parity(off, rowptr, col, val, A, B, what="gathered strips off")
 
 
+@pytest.mark.parametrize("K,dtype,n_dense_strips", [(32, "f32", 1), (32, "f32", 2), (64, "f32", 3), (64, "bf16", 2),
+                                                    (128, "f32", 1), (256, "f16", 2)])
+def test_gathered_pairs_behind_other_tiles(engine_factory, monkeypatch, K, dtype, n_dense_strips):
+    """Gathered strips come in pairs that share their B tiles (rows of up to 256 bytes: one
+    wavefront per two windows), and their descriptors start a window of their own: with 16-row
+    strips of fully dense tiles ahead of them whose tile count is not a multiple of four, the
+    window in between is filled with descriptors that stand for nothing.  Candidate counts of 1..3
+    strips and a half: a last pair without a second strip, and pairs whose two strips reach over
+    different tile columns."""
+    rng = np.random.default_rng(900 + K + n_dense_strips)
+    M, N = 16 * n_dense_strips + 700, 4000
+    rows = [np.sort(rng.choice(N, int(rng.integers(1, 10)), replace=False)) for _ in range(M)]
+    n_tiles_dense = 0
+    for sidx in range(n_dense_strips):                     # 16-row strips of 1, 2, 3 .. dense tiles: 1, 3, 6 in all
+        tcs = np.sort(rng.choice(N // 16, sidx + 1, replace=False))
+        cols = np.concatenate([16 * t + np.arange(16) for t in tcs])
+        for r in range(16 * sidx, 16 * sidx + 16):
+            rows[r] = cols.copy()
+        n_tiles_dense += len(tcs)
+    assert n_tiles_dense % 4 != 0
+    pool = np.arange(16 * n_dense_strips, M)
+    dense_rows = np.sort(rng.choice(pool, 16 * 3 + 9 + 32 * (K % 3), replace=False))
+    for r in dense_rows:
+        s0 = int(rng.choice([200, 1500, 1500, 2600]))
+        c = s0 + int(rng.integers(0, 40)) + np.nonzero(rng.random(500) < 0.55)[0]
+        rows[r] = np.unique(c)
+    lens = np.array([len(x) for x in rows])
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    if dtype == "bf16":
+        Ab, Bb = capi.to_bf16(A).reshape(M, K), capi.to_bf16(B).reshape(N, K)
+        A, B, ops, dt = capi.from_bf16(Ab).reshape(M, K), capi.from_bf16(Bb).reshape(N, K), (Ab, Bb), capi.BF16
+    elif dtype == "f16":
+        Ab, Bb = capi.to_f16(A).reshape(M, K), capi.to_f16(B).reshape(N, K)
+        A, B, ops, dt = capi.from_f16(Ab).reshape(M, K), capi.from_f16(Bb).reshape(N, K), (Ab, Bb), capi.F16
+    else:
+        ops, dt = (A, B), capi.F32
+    dense_nnz = int(lens[dense_rows].sum())
+    strips_nnz = int(lens[:16 * n_dense_strips].sum())
+    _say("gathered pairs", K, dtype, n_dense_strips)
+    got, st = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert_parity(got, rowptr, col, val, A, B, what="pairs behind %d dense tiles" % n_tiles_dense)
+    assert st.nnz_mfma >= strips_nnz + 0.6 * dense_nnz and st.mfma_tiles > n_tiles_dense
+    assert st.nnz_mfma + st.nnz_panel + st.nnz_short + st.nnz_medium + st.nnz_long == len(col)
+    # the same plan, one wavefront per window
+    monkeypatch.setenv("SDDMM_PAIRS", "0")
+    one, st1 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st1.mfma_tiles == st.mfma_tiles and st1.nnz_mfma == st.nnz_mfma
+    np.testing.assert_array_equal(one.view(np.uint32), got.view(np.uint32))
+    # and tile by tile from the descriptors
+    monkeypatch.setenv("SDDMM_WINDOW_FILL", "1")
+    walk, st2 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st2.mfma_tiles == st.mfma_tiles
+    assert_parity(walk, rowptr, col, val, A, B, what="pairs, tile by tile")
+
+
 def _host_union_model(M, rowptr, col, min_fill, span_limit=131072):
     """Union strips as the device must find them when no other path owns a row: a
     16-row strip is taken iff its rows are strictly increasing, its column span fits
