@@ -1398,6 +1398,147 @@ __global__ __launch_bounds__(BLOCK) void k_tile(const void *__restrict__ A, cons
                               blk * WAVES_PER_BLOCK + wave_in_block(), win_lds[wave_in_block()], order);
 }
 
+// ---- long rows, well-filled tiles: the four waves of a workgroup split K -----------------------
+// A tile of long rows is 16 KB of B (1 KiB rows) for 16 MFMAs: a wavefront that walks tiles alone has
+// two of them in flight, fills half the register file with them and still waits for memory most of
+// the time, and a launch of a few thousand tiles is two such wavefronts per SIMD.  Here a workgroup
+// takes one window of TILE_WINDOW tiles and wave j the j-th quarter of K of all of them: a quarter of
+// the registers per tile, all four tiles of the window in flight, four times the wavefronts.  The
+// partial 16x16 products meet in LDS (1 KiB per tile and wave); wave j then adds up tile j, scales it
+// by S and scatters it from the descriptor's masks, which it loaded at the start.
+constexpr int KSPLIT = WAVES_PER_BLOCK;
+static_assert(KSPLIT == 4 && TILE_WINDOW == 4, "one finishing wave per tile of a window");
+constexpr int KSPLIT_LDS_FLOATS = TILE_WINDOW * KSPLIT * 256;
+
+template <int DT, int STEPS>
+__global__ __launch_bounds__(BLOCK) void k_tile_ksplit(const void *__restrict__ A, const void *__restrict__ B, int M, int N,
+                                                       const int32_t *__restrict__ vrows,
+                                                       const int32_t *__restrict__ tile_cols,
+                                                       const TileDesc *__restrict__ tiles, int64_t n_tiles,
+                                                       const float *__restrict__ sval, float *__restrict__ P,
+                                                       int64_t nblocks, const int32_t *__restrict__ order) {
+    static_assert(STEPS % KSPLIT == 0, "K in four equal parts of whole 64-byte steps");
+    constexpr int SW = STEPS / KSPLIT;                    // steps of this wave
+    __shared__ __attribute__((aligned(16))) float part[KSPLIT_LDS_FLOATS];
+    int64_t w = xcd_remap(blockIdx.x, nblocks);
+    if (w < 0) return;                                    // whole workgroups leave
+    if (order) w = order[w];
+    const int64_t t0 = w * TILE_WINDOW;
+    if (t0 >= n_tiles) return;
+    const int n = (int)(n_tiles - t0 < TILE_WINDOW ? n_tiles - t0 : TILE_WINDOW);
+    const int j = wave_in_block();
+    const int lane = lane_id();
+    const int r16 = lane & 15, q = lane >> 4;        // operand / result layout
+    const int lrow = lane >> 2, lunit = lane & 3;    // memory layout: four neighbouring lanes on 64 bytes of a row
+    const int to_operand_from = (4 * r16 + q) << 2;
+    constexpr uint32_t ROW_UNITS = STEPS * 4;
+    const uint4 *__restrict__ Au = (const uint4 *)A + (uint32_t)(j * SW * 4);    // this wave's quarter of every row
+    const uint4 *__restrict__ Bu = (const uint4 *)B + (uint32_t)(j * SW * 4);
+    auto to_operand = [&](const uint4 &v) {
+        uint4 r;
+        r.x = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.x);
+        r.y = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.y);
+        r.z = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.z);
+        r.w = (uint32_t)__builtin_amdgcn_ds_bpermute(to_operand_from, (int)v.w);
+        return r;
+    };
+    // first round trip: strip and B rows of every tile, the per-row fields of this wave's own tile
+    // (one load each: lane u of every quad asks for tile u, the values are dealt out inside the quad)
+    int strip[TILE_WINDOW], bcol[TILE_WINDOW];
+    {
+        const int64_t t = t0 + (lunit < n ? lunit : n - 1);
+        const int st = tiles[t].strip;
+        const int bc = tile_cols[t * 16 + lrow];
+        strip[0] = __builtin_amdgcn_readlane(st, 0); strip[1] = __builtin_amdgcn_readlane(st, 1);
+        strip[2] = __builtin_amdgcn_readlane(st, 2); strip[3] = __builtin_amdgcn_readlane(st, 3);
+        bcol[0] = dpp_i32<0x00>(bc); bcol[1] = dpp_i32<0x55>(bc);       // quad_perm: every lane takes lane k of its quad
+        bcol[2] = dpp_i32<0xAA>(bc); bcol[3] = dpp_i32<0xFF>(bc);
+    }
+    const TileDesc *mine = tiles + t0 + (j < n ? j : n - 1);
+    const int4 off4 = *(const int4 *)&mine->off[q * 4];
+    const uint2 mask2 = *(const uint2 *)&mine->mask[q * 4];
+    auto a_rows = [&](int st) {
+        int64_t arow = st >= GATHERED_BASE ? (int64_t)vrows[(int64_t)(st - GATHERED_BASE) * 16 + lrow]
+                                           : (int64_t)st * 16 + lrow;
+        arow = arow < 0 ? 0 : (arow < M ? arow : M - 1);      // missing rows are never in a mask
+        return Au + arow * ROW_UNITS + lunit;
+    };
+    // second round trip: this wave's quarter of the A panel and of all B tiles, the S values of its own tile
+    uint4 a[SW], b[TILE_WINDOW][SW];
+    {
+        const uint4 *src = a_rows(strip[0]);
+#pragma unroll
+        for (int s = 0; s < SW; ++s) a[s] = src[s * 4];
+    }
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) {
+        int64_t brow = bcol[k];
+        brow = brow < N ? brow : N - 1;                   // columns past N (and the filler of a short union tile) are in no mask
+        const uint4 *src = Bu + brow * ROW_UNITS + lunit;
+#pragma unroll
+        for (int s = 0; s < SW; ++s) b[k][s] = src[s * 4];
+    }
+    const unsigned int below = (1u << r16) - 1u;
+    const int offs[4] = {off4.x, off4.y, off4.z, off4.w};
+    const unsigned int masks[4] = {mask2.x & 0xFFFFu, mask2.x >> 16, mask2.y & 0xFFFFu, mask2.y >> 16};
+    unsigned int act = 0;
+    int pos[4];
+    float sv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const bool on = j < n && ((masks[i] >> r16) & 1u);
+        act |= on ? (1u << i) : 0u;
+        pos[i] = on ? offs[i] + __builtin_popcount(masks[i] & below) : 0;   // (row 4q+i, column r16); entry 0 when absent
+        sv[i] = sval[pos[i]];
+    }
+#pragma unroll
+    for (int s = 0; s < SW; ++s) a[s] = to_operand(a[s]);
+#pragma unroll
+    for (int k = 0; k < TILE_WINDOW; ++k) {
+        if (k >= n) break;                                // workgroup-uniform
+        if (k > 0 && strip[k] != strip[k - 1]) {          // workgroup-uniform: the window reaches into the next strip
+            const uint4 *src = a_rows(strip[k]);
+#pragma unroll
+            for (int s = 0; s < SW; ++s) a[s] = to_operand(src[s * 4]);
+        }
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < SW; ++s) {
+            const uint4 bo = to_operand(b[k][s]);
+            if constexpr (DT == DT_BF16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a[s]),
+                                                              __builtin_bit_cast(bf16x8_t, bo), acc, 0, 0, 0);
+            } else if constexpr (DT == DT_F16) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a[s]),
+                                                             __builtin_bit_cast(half8_t, bo), acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].x),
+                                                           __builtin_bit_cast(float, bo.x), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].y),
+                                                           __builtin_bit_cast(float, bo.y), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].z),
+                                                           __builtin_bit_cast(float, bo.z), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s].w),
+                                                           __builtin_bit_cast(float, bo.w), acc, 0, 0, 0);
+            }
+        }
+        *reinterpret_cast<f32x4_t *>(part + (k * KSPLIT + j) * 256 + lane * 4) = acc;
+    }
+    __syncthreads();
+    if (j < n) {
+        f32x4_t sum = *reinterpret_cast<const f32x4_t *>(part + (j * KSPLIT) * 256 + lane * 4);
+#pragma unroll
+        for (int jj = 1; jj < KSPLIT; ++jj) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(part + (j * KSPLIT + jj) * 256 + lane * 4);
+            sum[0] += v[0]; sum[1] += v[1]; sum[2] += v[2]; sum[3] += v[3];
+        }
+        // result register i is row 4*q+i, column r16
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if ((act >> i) & 1u) P[pos[i]] = sum[i] * sv[i];
+    }
+}
+
 // Order of the windows for operands that exceed an XCD's L2.  The launch gives every XCD a
 // contiguous eighth of the logical windows (xcd_remap); sorted by the key below, that eighth is
 // one block of a RB x CB grid over (strip rows, tile columns), RB * CB = 8, walked by finer

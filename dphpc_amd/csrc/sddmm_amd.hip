@@ -964,6 +964,19 @@ void launch_panels(sddmm_ctx *c) {
 
 template <int DT, int STEPS>
 void launch_tile_t(sddmm_ctx *c) {
+    // Well-filled tiles (walked from the descriptors' masks) of rows of 256 bytes and more, fewer
+    // windows than keep the chip busy on their own: one workgroup per window, K in four parts.
+    if constexpr (STEPS % KSPLIT == 0) {
+        if (!c->use_windows && c->n_windows <= (int64_t)env_int("SDDMM_KSPLIT_MAX", 32768) && env_int("SDDMM_KSPLIT", 1) != 0) {
+            const int64_t nb = c->n_windows;
+            SDDMM_LAUNCH(c, (k_tile_ksplit<DT, STEPS>), xcd_grid(nb), BLOCK,
+                               (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
+                               (const int32_t *)c->d_tile_cols, (const TileDesc *)c->d_tiles, c->n_tiles,
+                               (const float *)c->d_sval, c->dP, nb,
+                               (const int32_t *)(c->use_win_order ? c->d_win_order : nullptr));
+            return;
+        }
+    }
     const int64_t nblocks = (c->n_tile_units + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
     SDDMM_LAUNCH(c, (k_tile<DT, STEPS>), xcd_grid(nblocks), BLOCK,
                        (const void *)c->dA, (const void *)c->dB, c->M, c->N, (const int32_t *)c->d_vrows,
