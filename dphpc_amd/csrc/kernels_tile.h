@@ -1875,26 +1875,26 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
     };
     struct Oper {
         uint4 b[STEPS];
-        F4u s;
     };
-    auto load_oper = [&](int cc, int u, int g0) {               // group u of the chunk whose columns are in cc
+    auto load_oper = [&](int cc, int u) {                       // group u of the chunk whose columns are in cc
         Oper o;
         const int c = __shfl(cc, u * 16 + lrow, WAVE);
         const uint4 *src = Bu + (int64_t)c * ROW_UNITS + lunit;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) o.b[s] = src[s * 4];
-        // The first group of a pair also brings the S values of entries g0+4*punit .. +3 of
-        // this lane's row, for both groups.  The window is clamped into the row (rows of a
-        // panel hold at least 4 entries); a clamped window is never used: lanes whose four
-        // entries are not all inside the item fetch their S values again.
-        o.s = F4u{0.f, 0.f, 0.f, 0.f};
-        if ((u & 1) == 0) {
-            int e = g0 + 4 * (punit - rot);
-            e = e < row_len - 4 ? e : row_len - 4;
-            e = e > 0 ? e : 0;
-            o.s = *reinterpret_cast<const F4u *>(sval + out_row + e);
-        }
         return o;
+    };
+    // The S values of entries g0+4*(punit-rot) .. +3 of this lane's row: one access for the pair of
+    // groups that starts at g0.  The window is clamped into the row (rows of a panel hold at
+    // least 4 entries); a clamped window is never used: lanes whose four entries are not all
+    // inside the item fetch their S values again.  (Requested one chunk ahead of its products;
+    // two chunks ahead was measured slower, in a loop 34 against 30 us and cold 53 against 48 us
+    // at 128-byte rows: a request that waits for HBM holds its place in the vector memory queue.)
+    auto load_s = [&](int g0) {
+        int e = g0 + 4 * (punit - rot);
+        e = e < row_len - 4 ? e : row_len - 4;
+        e = e > 0 ? e : 0;
+        return *reinterpret_cast<const F4u *>(sval + out_row + e);
     };
     auto permute4 = [&](int from, uint32_t x, uint32_t y, uint32_t z, uint32_t w_) {
         uint4 r;
@@ -1987,7 +1987,7 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
     };
     // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
     float held[4] = {0.f, 0.f, 0.f, 0.f};                        // ROTATE: the unit taken from the previous pair
-    auto compute_store_pair = [&](const Oper &o0, const Oper &o1, int g0) {
+    auto compute_store_pair = [&](const Oper &o0, const Oper &o1, const F4u &sw, int g0) {
         if (g0 >= end + (any_rot ? 32 : 0)) return;              // wave-uniform
         const bool past = g0 >= end;                             // the store-only step after the last pair
         float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
@@ -2038,7 +2038,7 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
             // ROTATE, first pair: these lanes' first unit comes with the next pair
         } else if (e + 4 <= end) {
             // four consecutive entries inside the item (so the S window was not clamped)
-            F4u out{d0 * o0.s.x, d1 * o0.s.y, d2 * o0.s.z, d3 * o0.s.w};
+            F4u out{d0 * sw.x, d1 * sw.y, d2 * sw.z, d3 * sw.w};
             *reinterpret_cast<F4u *>(P + out_row + e) = out;
             p[0] = out.x; p[1] = out.y; p[2] = out.z; p[3] = out.w;
         } else {
@@ -2073,12 +2073,14 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
     // this prologue too, so the prologue issues its loads in the order the loop does
     // (both column loads first, then the groups in the order they are consumed);
     // otherwise the loop would wait for almost everything it has just requested.
+    F4u s_cur[GROUPS / 2];
     const int cc0 = cols_of_chunk(start);
     int cc_nxt = cols_of_chunk(start + CHUNK);                  // columns of the next chunk
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < GROUPS; ++u) {
-        o[u] = load_oper(cc0, u, start + 16 * u);
+        o[u] = load_oper(cc0, u);
+        if ((u & 1) == 0) s_cur[u / 2] = load_s(start + 16 * u);
         __builtin_amdgcn_sched_barrier(0);
     }
     const int walk_end = end + (any_rot ? 32 : 0);
@@ -2086,9 +2088,10 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         const int cc_nn = cols_of_chunk(base + 2 * CHUNK);
 #pragma unroll
         for (int u = 0; u < GROUPS; u += 2) {
-            compute_store_pair(o[u], o[u + 1], base + 16 * u);
-            o[u] = load_oper(cc_nxt, u, base + CHUNK + 16 * u);
-            o[u + 1] = load_oper(cc_nxt, u + 1, base + CHUNK + 16 * u + 16);
+            compute_store_pair(o[u], o[u + 1], s_cur[u / 2], base + 16 * u);
+            o[u] = load_oper(cc_nxt, u);
+            o[u + 1] = load_oper(cc_nxt, u + 1);
+            s_cur[u / 2] = load_s(base + CHUNK + 16 * u);
         }
         cc_nxt = cc_nn;
     }
