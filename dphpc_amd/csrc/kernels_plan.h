@@ -332,6 +332,40 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_small(const unsigned int *_
     if (threadIdx.x == 0) *total_out = carry;
 }
 
+// Several short scans in one launch: workgroup j takes job j (in == out is allowed: a thread
+// writes only the positions it has read).
+constexpr int SCAN_JOBS_MAX = 8;
+struct ScanJob {
+    const unsigned int *in;
+    unsigned int *out;
+    unsigned long long *total;
+    int n;
+    int pad;
+};
+struct ScanJobs { ScanJob job[SCAN_JOBS_MAX]; };
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_jobs(ScanJobs jobs) {
+    const ScanJob jb = jobs.job[blockIdx.x];
+    unsigned int carry = 0;
+    for (int base = 0; base < jb.n; base += SCAN_BLOCK * SCAN_SMALL_ITEMS) {
+        const int i0 = base + (int)threadIdx.x * SCAN_SMALL_ITEMS;
+        unsigned int v[SCAN_SMALL_ITEMS], mine = 0;
+#pragma unroll
+        for (int q = 0; q < SCAN_SMALL_ITEMS; ++q) {
+            v[q] = i0 + q < jb.n ? jb.in[i0 + q] : 0u;
+            mine += v[q];
+        }
+        unsigned int total;
+        unsigned int at = carry + block_exclusive_scan(mine, &total);
+#pragma unroll
+        for (int q = 0; q < SCAN_SMALL_ITEMS; ++q) {
+            if (i0 + q < jb.n) jb.out[i0 + q] = at;
+            at += v[q];
+        }
+        carry += total;
+    }
+    if (threadIdx.x == 0) *jb.total = carry;
+}
+
 // The entry list of the short rows: {position, row} of every stored entry of the rows that
 // have fewer than ts entries and no owner, in storage order.  The kernels take it 64 entries
 // per wavefront, whatever the lengths of the rows (block_offsets: exclusive scan of the

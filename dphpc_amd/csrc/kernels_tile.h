@@ -155,7 +155,7 @@ __device__ __forceinline__ void write_aligned_cols(int32_t *__restrict__ tile_co
 // order, so clearing, marking and counting need no workgroup barrier, only that
 // the compiler keeps their order (wave_lds_order).
 constexpr int STRIP_BM_WORDS = 1024;          // 32768 tile columns: a span of 524288 columns
-constexpr int STRIP_UNROLL = 8;               // loads of 64 entries per batch, two batches in flight
+constexpr int STRIP_UNROLL = 4;               // loads of 256 entries per batch, two batches in flight
 constexpr int STRIPS_PER_BLOCK = 4;
 
 __device__ __forceinline__ void wave_lds_order() {
@@ -163,49 +163,78 @@ __device__ __forceinline__ void wave_lds_order() {
     __builtin_amdgcn_wave_barrier();
 }
 
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
 // Streams entries [e0, e1).  Returns the number of tile-column changes, or -1 as
 // soon as it exceeds `budget`; *descents receives the number of entries whose
 // column does not exceed the column stored before them.  BITS == 1: also sets bit
 // (col>>4) - lo in bm after every change (tile columns); BITS == 2: sets bit col - lo
 // for every entry (columns).
+// A lane takes four consecutive entries per load (16 bytes; the column array is only
+// 4-byte aligned at a strip's start, which global loads allow), a load instruction 256
+// entries, a batch STRIP_UNROLL of them with the next batch in flight: a strip of 8 000
+// entries is eight dependent round trips.
 template <int BITS>
 __device__ __forceinline__ int64_t strip_scan(const int32_t *__restrict__ col, int e0, int e1, int64_t budget,
                                               int lo, int span, unsigned int *bm, int64_t *descents) {
     const int lane = lane_id();
-    constexpr int BATCH = WAVE * STRIP_UNROLL;
+    constexpr int PER_LOAD = WAVE * 4;
+    constexpr int BATCH = PER_LOAD * STRIP_UNROLL;
     int64_t changes = 0, desc = 0;
     int carry = -1;                           // column before the batch; -1: entry e0 counts as a change
-    auto load = [&](int base, int (&c)[STRIP_UNROLL]) {
+    auto load = [&](int base, I4u (&c)[STRIP_UNROLL]) {
 #pragma unroll
         for (int u = 0; u < STRIP_UNROLL; ++u) {
-            const int e = base + u * WAVE + lane;
-            if (base + u * WAVE < e1 || u == 0) c[u] = col[e < e1 ? e : e1 - 1];   // wave-uniform skip
-            else c[u] = 0;
+            const int b = base + u * PER_LOAD;
+            if (b + PER_LOAD <= e1) {                             // wave-uniform: every lane's four entries exist
+                c[u] = *reinterpret_cast<const I4u *>(col + b + 4 * lane);
+            } else if (b < e1 || u == 0) {                        // the last load of the strip: clamped, entry by entry
+                const int last = e1 - 1, i0 = b + 4 * lane;
+                c[u].x = col[i0 < last ? i0 : last];
+                c[u].y = col[i0 + 1 < last ? i0 + 1 : last];
+                c[u].z = col[i0 + 2 < last ? i0 + 2 : last];
+                c[u].w = col[i0 + 3 < last ? i0 + 3 : last];
+            } else {
+                c[u] = I4u{0, 0, 0, 0};
+            }
         }
     };
-    int cur[STRIP_UNROLL], nxt[STRIP_UNROLL];
+    auto mark = [&](bool on, int column) {
+        if constexpr (BITS == 1) {
+            const int t = (column >> 4) - lo;
+            if (on && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
+        } else if constexpr (BITS == 2) {
+            const int t = column - lo;
+            if (on && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
+        }
+    };
+    I4u cur[STRIP_UNROLL], nxt[STRIP_UNROLL];
     load(e0, cur);
     for (int base = e0; base < e1; base += BATCH) {
         load(base + BATCH, nxt);
+        int my_changes = 0, my_desc = 0;
 #pragma unroll
         for (int u = 0; u < STRIP_UNROLL; ++u) {
-            const int cbase = base + u * WAVE;
-            if (cbase >= e1) break;                           // wave-uniform
-            const bool valid = cbase + lane < e1;
-            // column of the entry before: lane - 1 (wave_shr:1), lane 0 takes the carry
-            const int prev = __builtin_amdgcn_update_dpp(carry, cur[u], 0x138, 0xF, 0xF, false);
-            carry = __builtin_amdgcn_readlane(cur[u], WAVE - 1);
-            const bool change = valid && (cur[u] >> 4) != (prev >> 4);
-            if constexpr (BITS == 1) {
-                const int t = (cur[u] >> 4) - lo;
-                if (change && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
-            } else if constexpr (BITS == 2) {
-                const int t = cur[u] - lo;
-                if (valid && (unsigned int)t < (unsigned int)span) atomicOr(&bm[t >> 5], 1u << (t & 31));
-            }
-            changes += __popcll(__ballot(change));
-            desc += __popcll(__ballot(valid && cur[u] <= prev));
+            const int cbase = base + u * PER_LOAD;
+            if (cbase >= e1) break;                               // wave-uniform
+            const int i0 = cbase + 4 * lane;
+            const I4u c = cur[u];
+            // column of the entry before this lane's first: the last of lane - 1 (wave_shr:1), lane 0 takes the carry
+            const int prev = __builtin_amdgcn_update_dpp(carry, c.w, 0x138, 0xF, 0xF, false);
+            carry = __builtin_amdgcn_readlane(c.w, WAVE - 1);
+            const bool v0 = i0 < e1, v1 = i0 + 1 < e1, v2 = i0 + 2 < e1, v3 = i0 + 3 < e1;
+            const bool c0 = v0 && (c.x >> 4) != (prev >> 4), c1 = v1 && (c.y >> 4) != (c.x >> 4);
+            const bool c2 = v2 && (c.z >> 4) != (c.y >> 4), c3 = v3 && (c.w >> 4) != (c.z >> 4);
+            if constexpr (BITS == 1) { mark(c0, c.x); mark(c1, c.y); mark(c2, c.z); mark(c3, c.w); }
+            if constexpr (BITS == 2) { mark(v0, c.x); mark(v1, c.y); mark(v2, c.z); mark(v3, c.w); }
+            my_changes += (int)c0 + (int)c1 + (int)c2 + (int)c3;
+            my_desc += (int)(v0 && c.x <= prev) + (int)(v1 && c.y <= c.x) + (int)(v2 && c.z <= c.y) + (int)(v3 && c.w <= c.z);
         }
+        changes += wave_sum_i32(my_changes);
+        desc += wave_sum_i32(my_desc);
         if (changes > budget) return -1;
 #pragma unroll
         for (int u = 0; u < STRIP_UNROLL; ++u) cur[u] = nxt[u];
@@ -236,11 +265,6 @@ __device__ __forceinline__ void strip_bounds(const int32_t *__restrict__ col, in
     *boundary_descents = __popcll(__ballot(has && first_col <= before));
 }
 
-__device__ __forceinline__ int wave_sum_i32(int v) {
-    for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
-}
-
 // pass 1: strip_ntiles[s] = number of tiles of a strip that goes to the tile path
 // (sorted rows, at least min_fill entries per tile on average), else 0.
 __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
@@ -262,7 +286,7 @@ __global__ __launch_bounds__(WAVE * STRIPS_PER_BLOCK) void k_strip_count(
     bool take = false;
     // most strips of a scattered matrix are given up on their first 512 entries,
     // before anything else is read
-    constexpr int FIRST = WAVE * STRIP_UNROLL;
+    constexpr int FIRST = 512;
     if (max_tiles > 0 &&
         strip_scan<0>(col, e0, e1 - e0 > FIRST ? e0 + FIRST : e1, budget, 0, 0, nullptr, &descents) >= 0) {
         int lo, span, allowed;

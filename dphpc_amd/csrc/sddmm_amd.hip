@@ -111,6 +111,8 @@ struct sddmm_ctx {
     int64_t panels_cap = 0;
     int2 *d_short_list = nullptr;    // {position, row} of the entries of the short rows nobody owns
     int64_t n_short_list = 0, short_list_cap = 0;
+    ScanJobs scan_jobs{};            // short scans waiting for the next read-back of the counters
+    int n_scan_jobs = 0;
     bool use_short_list = false;
     unsigned int *d_short_sums = nullptr;   // arena view: entries of short rows per block of the row scan
     RowItem *d_panel_items = nullptr;
@@ -309,7 +311,30 @@ int grid_capped(int64_t n, int block, int cap = 16384) {
     return (int)std::min<int64_t>(cap, std::max<int64_t>(1, (n + block - 1) / block));
 }
 
+// The short scans of a plan (tiles per strip, items per panel, block sums of the row classes ...) feed
+// nothing before the next read-back of the counters, so they are collected and run as ONE launch
+// there instead of one launch each behind its producer.
+int flush_scans(sddmm_ctx *c) {
+    if (c->n_scan_jobs == 0) return SDDMM_OK;
+    SDDMM_LAUNCH(c, k_scan_jobs, c->n_scan_jobs, SCAN_BLOCK, c->scan_jobs);
+    c->n_scan_jobs = 0;
+    LAUNCH_CHECK(c);
+    return SDDMM_OK;
+}
+int queue_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t n, unsigned long long *d_total) {
+    if (c->n_scan_jobs == SCAN_JOBS_MAX) {
+        const int rc = flush_scans(c);
+        if (rc) return rc;
+    }
+    c->scan_jobs.job[c->n_scan_jobs++] = ScanJob{in, out, d_total, (int)n, 0};
+    return SDDMM_OK;
+}
+
 int fetch_counters(sddmm_ctx *c) {
+    {
+        const int rc = flush_scans(c);
+        if (rc) return rc;
+    }
     HIP_TRY(c, hipMemcpyAsync(c->h_pc, c->d_pc, sizeof(DevCounters), hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(c, hipStreamSynchronize(c->stream));
     c->raw = *c->h_pc;
@@ -526,11 +551,19 @@ int classify_rows_count(sddmm_ctx *c, bool again = false) {
         const unsigned char *owner = c->owner_active ? c->d_owner : nullptr;
         SDDMM_LAUNCH(c, k_classify_count, nb, SCAN_BLOCK, c->d_rowptr, owner,
                            c->sM, c->ts, c->seg, c->d_block_sums, c->d_pc, 0, c->d_short_sums);
-        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
-                           &c->d_pc->n_items);
-        SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_short_sums, (int)nb,
-                           &c->d_pc->short_scanned);
         LAUNCH_CHECK(c);
+        if (nb <= SCAN_SMALL_MAX) {
+            int rc = queue_scan(c, c->d_block_sums, c->d_block_sums, nb, &c->d_pc->n_items);
+            if (rc) return rc;
+            rc = queue_scan(c, c->d_short_sums, c->d_short_sums, nb, &c->d_pc->short_scanned);
+            if (rc) return rc;
+        } else {
+            SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_block_sums, (int)nb,
+                               &c->d_pc->n_items);
+            SDDMM_LAUNCH(c, k_scan_block_sums, 1, SCAN_BLOCK, c->d_short_sums, (int)nb,
+                               &c->d_pc->short_scanned);
+            LAUNCH_CHECK(c);
+        }
     }
     return SDDMM_OK;
 }
@@ -589,10 +622,10 @@ int classify_rows_items(sddmm_ctx *c, bool with_short_list = true) {
 
 // Exclusive scan of n unsigned ints on the device (in != out), total to *d_total.
 int device_scan(sddmm_ctx *c, const unsigned int *in, unsigned int *out, int64_t n, unsigned long long *d_total) {
-    if (n <= SCAN_SMALL_MAX) {
-        SDDMM_LAUNCH(c, k_scan_small, 1, SCAN_BLOCK, in, (int)n, out, d_total);
-        LAUNCH_CHECK(c);
-        return SDDMM_OK;
+    if (n <= SCAN_SMALL_MAX) return queue_scan(c, in, out, n, d_total);
+    {
+        const int rc = flush_scans(c);             // (the long scan borrows the block sums)
+        if (rc) return rc;
     }
     const int64_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
     ARENA_HOLDS(c, nb, c->block_sums_cap, "block sums");
@@ -1091,6 +1124,7 @@ int do_plan(sddmm_ctx *c, int strategy) {
     // the plan state is rewritten in place: a plan that fails half way must not leave the
     // previous one looking valid (its items exclude rows that tiles and panels owned)
     c->planned = false;
+    c->n_scan_jobs = 0;
     c->fused_items_valid = false;    // they leave out the rows of this plan's panels
     int resolved = strategy;
     const bool csr_ok = c->have_rowptr;
