@@ -239,6 +239,38 @@ def fused_leg(e, w, capi, reps, check):
             log("VALIDATION FAILED (fused): element %d got %r (%.2f x tolerance)" % (i, got[:w.M].ravel()[i], worst))
             sys.exit(1)
         res["validated"] = {"elements": int(w.M * w.K), "worst_over_tol": round(worst, 4)}
+    if w.dtype == "f32" and w.K % 8 == 0:
+        res["bf16_operands"] = fused_bf16_leg(w, capi, reps, check)
+    return res
+
+
+def fused_bf16_leg(w, capi, reps, check):
+    """The same fused call with A and B stored as bfloat16 (P and O stay fp32), validated
+    against the fp32 oracle on the rounded operands."""
+    Ab, Bb = capi.to_bf16(w.A).reshape(w.A.shape), capi.to_bf16(w.B).reshape(w.B.shape)
+    e = capi.Engine(0)
+    e.set_dense(Ab, Bb, capi.BF16)
+    e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
+    e.plan(capi.AUTO)
+    times = []
+    for _ in range(reps):
+        e.run_fused(fetch=False)
+        times.append(e.stats().run_ms)
+    t = float(np.median(times))
+    res = {"ms_p50": t, "ms_min": float(min(times)), "gflops": 4.0 * w.nnz * w.K / (t * 1e-3) / 1e9,
+           "kernels_launched": e.stats().kernels_launched, "validated": None}
+    if check:
+        from oracle import oracle as O
+        got = e.run_fused()
+        Ar, Br = capi.from_bf16(Ab).reshape(w.A.shape), capi.from_bf16(Bb).reshape(w.B.shape)
+        _, ref_o = O.fusedmm_csr(w.rowptr, w.col, w.sval, Ar, Br)
+        _, mag_o = O.fusedmm_csr_f64(w.rowptr, w.col, w.sval, Ar, Br)
+        ok, worst, i = O.check_values_fast(got[:w.M].ravel(), ref_o.ravel(), mag=mag_o.ravel(), rtol=1e-5)
+        if not ok:
+            log("VALIDATION FAILED (fused, bf16 operands): element %d got %r (%.2f x tolerance)" % (i, got[:w.M].ravel()[i], worst))
+            sys.exit(1)
+        res["validated"] = {"elements": int(w.M * w.K), "worst_over_tol": round(worst, 4)}
+    e.close()
     return res
 
 

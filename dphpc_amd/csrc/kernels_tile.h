@@ -1800,7 +1800,7 @@ __device__ __forceinline__ void quad_transpose(float (&f)[4], int lane) {
 // with 2 than with 4 at rows of 128-256 bytes, 2-5 % slower at 512 bytes.
 constexpr int panel_mfma_waves(int steps) { return steps <= 4 ? 2 : 4; }
 
-// FUSED (fp32, rows of 128 or 256 bytes): the kernel also adds the panel's part of
+// FUSED (rows of 128 to 512 bytes in fp32, 64 to 256 bytes in bf16 / fp16): the kernel also adds the panel's part of
 //
 //     O[row0+r][:] += sum over the item's columns c of P[row0+r][c] * B[col_c][:]
 //
@@ -1813,25 +1813,30 @@ constexpr int panel_mfma_waves(int steps) { return steps <= 4 ? 2 : 4; }
 // the last column the 16 blocks are added with lane swaps and row rotations and every
 // lane adds 2*STEPS values to O atomically (O is cleared before the launch; a row may
 // be cut into several items).  Columns past the end of the item enter with srcB = 0,
-// whatever their B rows hold.
+// whatever their B rows hold.  16-bit operands: a B unit holds 8 components, widened to fp32 for
+// the second product (P and O are fp32 whatever the operands are), so there are 8 accumulators
+// per (h, s) and register i of lane 4b+j of accumulator (h,s,comp) collects O[4h+i][32s+8j+comp].
 constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;   // rotation by 4 / 8 lanes inside every row of 16
 constexpr int PANEL_TILE_PITCH = 48;                        // floats per row of the P tile: conflict-free 4-byte reads
 
-// waves per SIMD the register allocation aims at: the fused kernel keeps 32 * STEPS accumulators of
-// the output rows (3 waves at 128-byte rows -- 4 were no faster --, 2 at 256 bytes, measured 89 us
-// against 114 us with 1; at 512 bytes the accumulators leave room for one)
-constexpr int panel_mfma_min_waves(int steps, bool fused) {
-    return fused ? (steps == 2 ? 3 : steps == 4 ? 2 : 1) : steps == 8 ? 4 : 1;
+// waves per SIMD the register allocation aims at: the fused kernel keeps 2 * K accumulators of the
+// output rows, K = 16 * STEPS in fp32 and 32 * STEPS in 16 bits (3 waves at K = 32 -- 4 were no
+// faster --, 2 at K = 64, measured 89 us against 114 us with 1; at K = 128 the accumulators leave
+// room for one)
+constexpr int panel_mfma_min_waves(int steps, bool fused, bool half_width = false) {
+    const int k = steps * (half_width ? 32 : 16);
+    return fused ? (k <= 32 ? 3 : k == 64 ? 2 : 1) : steps == 8 ? 4 : 1;
 }
 
 template <int DT, int STEPS, bool FUSED = false>
-__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_waves(STEPS, FUSED)) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
+__global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_waves(STEPS, FUSED, DT != DT_F32)) void k_panel_mfma(const void *__restrict__ A, const void *__restrict__ B,
                                                       const int32_t *__restrict__ rowptr,
                                                       const int32_t *__restrict__ col,
                                                       const float *__restrict__ sval, float *__restrict__ P,
                                                       const RowItem *__restrict__ items, int64_t n_items,
                                                       int64_t nblocks, float *__restrict__ O) {
-    static_assert(!FUSED || (DT == DT_F32 && (STEPS == 2 || STEPS == 4 || STEPS == 8)), "fused panels: fp32 rows of 128 to 512 bytes");
+    static_assert(!FUSED || (DT == DT_F32 ? (STEPS == 2 || STEPS == 4 || STEPS == 8) : (STEPS == 1 || STEPS == 2 || STEPS == 4)),
+                  "fused panels: 32, 64 or 128 components per row");
     __shared__ __attribute__((aligned(16))) float p_tiles[FUSED ? panel_mfma_waves(STEPS) : 1][FUSED ? PANEL_ROWS * PANEL_TILE_PITCH : 4];
     const int64_t blk = xcd_remap(blockIdx.x, nblocks);
     if (blk < 0) return;
@@ -1982,14 +1987,15 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         return acc;
     };
     // FUSED: accumulator (h, s, comp) of the output rows, see above
-    f32x4_t oacc[2][STEPS][4];
+    constexpr int COMPS = DT == DT_F32 ? 4 : 8;                 // components of a 16-byte unit
+    f32x4_t oacc[2][STEPS][COMPS];
     if constexpr (FUSED) {
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) oacc[h][s][k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                for (int k = 0; k < COMPS; ++k) oacc[h][s][k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
     auto fused_accumulate = [&](const Oper &o, float p_lo, float p_hi, int gbase) {
         const bool live = gbase + lrow < end;                    // this block's column belongs to the item
@@ -1997,16 +2003,20 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         for (int s = 0; s < (FUSED ? STEPS : 0); ++s) {
             const uint4 b = o.b[s];
             const unsigned int ux = live ? b.x : 0u, uy = live ? b.y : 0u, uz = live ? b.z : 0u, uw = live ? b.w : 0u;
-            const float bx = __builtin_bit_cast(float, ux), by = __builtin_bit_cast(float, uy);
-            const float bz = __builtin_bit_cast(float, uz), bw = __builtin_bit_cast(float, uw);
-            oacc[0][s][0] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bx, oacc[0][s][0], 0, 0, 0);
-            oacc[1][s][0] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bx, oacc[1][s][0], 0, 0, 0);
-            oacc[0][s][1] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, by, oacc[0][s][1], 0, 0, 0);
-            oacc[1][s][1] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, by, oacc[1][s][1], 0, 0, 0);
-            oacc[0][s][2] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bz, oacc[0][s][2], 0, 0, 0);
-            oacc[1][s][2] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bz, oacc[1][s][2], 0, 0, 0);
-            oacc[0][s][3] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bw, oacc[0][s][3], 0, 0, 0);
-            oacc[1][s][3] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bw, oacc[1][s][3], 0, 0, 0);
+            float bv[COMPS];
+            if constexpr (DT == DT_F32) {
+                bv[0] = __builtin_bit_cast(float, ux); bv[1] = __builtin_bit_cast(float, uy);
+                bv[2] = __builtin_bit_cast(float, uz); bv[3] = __builtin_bit_cast(float, uw);
+            } else {
+                using U16 = std::conditional_t<DT == DT_BF16, UnitBF16x8, UnitF16x8>;
+                bv[0] = U16::lo(ux); bv[1] = U16::hi(ux); bv[2] = U16::lo(uy); bv[3] = U16::hi(uy);
+                bv[4] = U16::lo(uz); bv[5] = U16::hi(uz); bv[6] = U16::lo(uw); bv[7] = U16::hi(uw);
+            }
+#pragma unroll
+            for (int k = 0; k < COMPS; ++k) {
+                oacc[0][s][k] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_lo, bv[k], oacc[0][s][k], 0, 0, 0);
+                oacc[1][s][k] = __builtin_amdgcn_mfma_f32_4x4x1f32(p_hi, bv[k], oacc[1][s][k], 0, 0, 0);
+            }
         }
     };
     // groups o0 (entries g0..g0+15) and o1 (g0+16..g0+31) of the shared column list
@@ -2120,30 +2130,33 @@ __global__ __launch_bounds__(panel_mfma_waves(STEPS) * WAVE, panel_mfma_min_wave
         cc_nxt = cc_nn;
     }
     if constexpr (FUSED) {
-        // Register i of lane 4b+j of accumulator (h,s,comp) is O[4h+i][16s+4j+comp] over block b's
-        // columns.  The swaps add the four rows of 16 lanes while dealing the registers out: row r
+        // Register i of lane 4b+j of accumulator (h,s,comp) is O[4h+i][(4s+j) COMPS + comp] over block
+        // b's columns.  The swaps add the four rows of 16 lanes while dealing the registers out: row r
         // of the wave keeps register {0,2,1,3}[r]; the rotations add the four blocks of a row.  All
-        // four blocks then hold the same 16 sums; block cg adds the ones of component cg to O.
+        // four blocks then hold the same 16 sums; block cg adds the ones of components cg (and 4+cg) to O.
         const int r16 = lane >> 4, cg = (lane >> 2) & 3;
         const int orow = row0 + ((r16 & 1) << 1 | (r16 >> 1));
-        constexpr int K = STEPS * 16;
+        constexpr int K = STEPS * 4 * COMPS;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
-                float w4[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const f32x4_t v = oacc[h][s][k];
-                    const float t0 = swap32_add(v[0], v[1]);
-                    const float t1 = swap32_add(v[2], v[3]);
-                    float x = swap16_add(t0, t1);
-                    x += dpp_f32<DPP_ROW_ROR4>(x);
-                    x += dpp_f32<DPP_ROW_ROR8>(x);
-                    w4[k] = x;
+                for (int c4 = 0; c4 < COMPS; c4 += 4) {
+                    float w4[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const f32x4_t v = oacc[h][s][c4 + k];
+                        const float t0 = swap32_add(v[0], v[1]);
+                        const float t1 = swap32_add(v[2], v[3]);
+                        float x = swap16_add(t0, t1);
+                        x += dpp_f32<DPP_ROW_ROR4>(x);
+                        x += dpp_f32<DPP_ROW_ROR8>(x);
+                        w4[k] = x;
+                    }
+                    const float mine = cg == 0 ? w4[0] : cg == 1 ? w4[1] : cg == 2 ? w4[2] : w4[3];
+                    atomicAdd(O + (int64_t)(orow + 4 * h) * K + (4 * s + (lane & 3)) * COMPS + c4 + cg, mine);
                 }
-                const float mine = cg == 0 ? w4[0] : cg == 1 ? w4[1] : cg == 2 ? w4[2] : w4[3];
-                atomicAdd(O + (int64_t)(orow + 4 * h) * K + 16 * s + 4 * (lane & 3) + cg, mine);
             }
         }
     }

@@ -963,11 +963,11 @@ void launch_panel_mfma_t(sddmm_ctx *c) {
                        c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks, (float *)nullptr);
 }
 // the panels of the fused SDDMM+SpMM: P and the panels' part of O
-template <int STEPS>
+template <int DT, int STEPS>
 void launch_panel_fused_t(sddmm_ctx *c) {
     constexpr int PW = panel_mfma_waves(STEPS);
     const int64_t nblocks = (c->n_panel_items + PW - 1) / PW;
-    SDDMM_LAUNCH(c, (k_panel_mfma<DT_F32, STEPS, true>), xcd_grid(nblocks), PW * WAVE,
+    SDDMM_LAUNCH(c, (k_panel_mfma<DT, STEPS, true>), xcd_grid(nblocks), PW * WAVE,
                        (const void *)c->dA, (const void *)c->dB, c->d_rowptr, c->d_col, (const float *)c->d_sval,
                        c->dP, (const RowItem *)c->d_panel_items, c->n_panel_items, nblocks, c->dO);
 }
@@ -1661,10 +1661,10 @@ int sddmm_run_fused(sddmm_ctx *c) {
         return fail(c, SDDMM_ERR_UNSUPPORTED,
                     "the fused SDDMM+SpMM needs K <= 256, a multiple of 4 (fp32) or 8 (bf16, fp16)");
     if (!c->have_rowptr) return fail(c, SDDMM_ERR_UNSUPPORTED, "the fused SDDMM+SpMM needs row-sorted entries");
-    // fp32 rows of 128 or 256 bytes: the 8-row panels of the current plan (AUTO if there is none
+    // rows of 32, 64 or 128 components: the 8-row panels of the current plan (AUTO if there is none
     // yet) take the matrix-core kernel, which shares every gathered B row between 8 rows and both
     // products; the other rows take the gather kernels
-    bool panels = c->dtype == SDDMM_F32 && (c->K == 32 || c->K == 64 || c->K == 128) && env_int("SDDMM_FUSED_PANELS", 1) != 0;
+    bool panels = (c->K == 32 || c->K == 64 || c->K == 128) && env_int("SDDMM_FUSED_PANELS", 1) != 0;
     if (panels && !c->planned) {
         rc = sddmm_plan(c, c->requested);
         if (rc) return rc;
@@ -1709,9 +1709,19 @@ int sddmm_run_fused(sddmm_ctx *c) {
             }
         });
         if (panels) {
-            if (c->K == 32) launch_panel_fused_t<2>(c);
-            else if (c->K == 64) launch_panel_fused_t<4>(c);
-            else launch_panel_fused_t<8>(c);
+            if (c->dtype == SDDMM_F32) {
+                if (c->K == 32) launch_panel_fused_t<DT_F32, 2>(c);
+                else if (c->K == 64) launch_panel_fused_t<DT_F32, 4>(c);
+                else launch_panel_fused_t<DT_F32, 8>(c);
+            } else if (c->dtype == SDDMM_BF16) {
+                if (c->K == 32) launch_panel_fused_t<DT_BF16, 1>(c);
+                else if (c->K == 64) launch_panel_fused_t<DT_BF16, 2>(c);
+                else launch_panel_fused_t<DT_BF16, 4>(c);
+            } else {
+                if (c->K == 32) launch_panel_fused_t<DT_F16, 1>(c);
+                else if (c->K == 64) launch_panel_fused_t<DT_F16, 2>(c);
+                else launch_panel_fused_t<DT_F16, 4>(c);
+            }
             ++launches;
         }
         LAUNCH_CHECK(c);

@@ -227,6 +227,61 @@ def test_fused_row_panels_on_the_matrix_cores(engine_factory, monkeypatch, K, st
     e.close()
 
 
+def _rounded(A, dtype):
+    """(stored 16-bit array, the fp32 values it holds)"""
+    if dtype == capi.BF16:
+        h = capi.to_bf16(A).reshape(A.shape)
+        return h, capi.from_bf16(h).reshape(A.shape)
+    h = capi.to_f16(A).reshape(A.shape)
+    return h, capi.from_f16(h).reshape(A.shape)
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("K", [32, 64, 128])
+def test_fused_row_panels_of_16bit_operands(engine_factory, monkeypatch, K, dtype):
+    """bf16 / fp16 rows of 64 / 128 / 256 bytes: the panels take the panel kernel here too (the B
+    units widened to fp32 for the second product), against the fp32 oracle on the rounded operands.
+    One panel's list ends on an infinite B row right after an item boundary."""
+    monkeypatch.setenv("SDDMM_PANEL_SEG", "128")
+    rng = np.random.default_rng(5200 + K + dtype)
+    N = 1500
+    panel_lens = [4, 5, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300, 700]
+    loose = [[0, 3, 70, 1, 0, 200, 9, 64]] * 5 + [[12] * 8] * 3
+    M, rowptr, col = _panel_pattern(rng, N, panel_lens, loose)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    Ah, Ar = _rounded(rng.uniform(-1, 1, (M, K)).astype(f32), dtype)
+    Bh, Br = _rounded(rng.uniform(-1, 1, (N, K)).astype(f32), dtype)
+    e = engine_factory()
+    e.set_dense(Ah, Bh, dtype)
+    e.set_csr(M, N, rowptr, col, val)
+    e.plan(capi.AUTO)
+    _check(e, rowptr, col, val, Ar, Br, "16-bit panels K=%d dtype=%d" % (K, dtype))
+    assert e.stats().kernels_launched == 3               # short rows, long rows, panels
+    monkeypatch.setenv("SDDMM_FUSED_PANELS", "0")
+    _check(e, rowptr, col, val, Ar, Br, "16-bit panels off")
+    assert e.stats().kernels_launched == 2
+    monkeypatch.delenv("SDDMM_FUSED_PANELS")
+    # panels only, a list of 129 columns whose last B row holds an infinity: the other panels stay finite
+    M2, rowptr2, col2 = _panel_pattern(rng, N - 1, [129, 40, 129], [])
+    col2 = col2.copy()
+    for r in range(8):
+        col2[rowptr2[r] + 128] = N - 1
+    val2 = rng.uniform(-1, 1, len(col2)).astype(f32)
+    Br2 = Br.copy(); Br2[N - 1, K - 3] = np.inf
+    Bh2, Br2 = _rounded(Br2, dtype)
+    e.set_dense(Ah[:M2].copy(), Bh2, dtype)
+    e.set_csr(M2, N, rowptr2, col2, val2)
+    e.plan(capi.AUTO)
+    got_o = e.run_fused()
+    assert e.stats().kernels_launched == 1
+    with np.errstate(all="ignore"):
+        _, ref_o = O.fusedmm_csr(rowptr2, col2, val2, Ar[:M2], Br2)
+    assert np.array_equal(np.isfinite(got_o[:M2]), np.isfinite(ref_o))
+    assert np.isfinite(got_o[8:M2]).all() and not np.isfinite(got_o[:8]).all()
+    np.testing.assert_allclose(got_o[8:M2], ref_o[8:], rtol=1e-4, atol=1e-5)
+    e.close()
+
+
 def test_fused_row_panels_keep_non_finite_b_rows_in_their_own_entries(engine_factory, monkeypatch):
     """A panel's list is cut into items of 128 columns and ends in the middle of a group of 16:
     the groups past an item's end load the B row of a clamped position, and the first column of
