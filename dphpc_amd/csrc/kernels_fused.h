@@ -56,58 +56,105 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[i][e] = 0.f;
     const int last = end - 1;
-    for (int base = start; base < end; base += WAVE) {
-        const int n = base + lane;
-        const bool valid = n < end;
-        const int c = col[n < last ? n : last];
-        const float s = valid ? sval[n] : 0.f;        // entries past the end contribute p = 0
-        const Off_t boff = (Off_t)c * rb;
-        const int count = end - base < WAVE ? end - base : WAVE;
-        int steps = (count + G - 1) / G;
-        steps = steps < LPN ? steps : LPN;
-        float out = 0.f;
-        for (int t0 = 0; t0 < steps; t0 += NB) {
-            T bf[NB][UPL];
+    struct Ent { int n, c; float s; bool valid; };
+    auto entry = [&](int base) {                      // entry base + lane of the item (clamped past its end)
+        Ent x;
+        x.n = base + lane;
+        x.valid = x.n < end;
+        x.c = col[x.n < last ? x.n : last];
+        x.s = x.valid ? sval[x.n] : 0.f;              // entries past the end contribute p = 0
+        return x;
+    };
+    // steps t0 .. t0+NB-1 of a chunk: group g gathers the B rows of entries t*G+g
+    auto gather = [&](const Ent &x, int t0, T (&bf)[NB][UPL]) {
+        const Off_t boff = (Off_t)x.c * rb;
 #pragma unroll
-            for (int q = 0; q < NB; ++q) {
-                const int src = ((t0 + q) * G + g) & (WAVE - 1);
-                const Off_t bo = shfl_off<Off_t>(boff, src);
+        for (int q = 0; q < NB; ++q) {
+            const int src = ((t0 + q) * G + g) & (WAVE - 1);
+            const Off_t bo = shfl_off<Off_t>(boff, src);
 #pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
-                    bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
-                }
-            }
-#pragma unroll
-            for (int q = 0; q < NB; ++q) {
-                if (t0 + q >= steps) break;               // wave-uniform
-                const int src = ((t0 + q) * G + g) & (WAVE - 1);
-                float p = 0.f;
-#pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    const float d = U::dot(a.u[i], bf[q][i], p);
-                    p = C::unit_on(j, i, KU) ? d : p;
-                }
-                // a step past the end of the row works on a clamped position: it must leave the
-                // output row alone whatever that position's B row holds (0 * inf is not 0)
-                const bool live = __shfl((int)valid, src, WAVE) != 0;
-                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);     // every lane takes part in the lane exchange
-                p = live ? p : 0.f;
-#pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    float next[E];
-#pragma unroll
-                    for (int e = 0; e < E; ++e) next[e] = acc[i][e];
-                    U::axpy(p, bf[q][i], next);
-#pragma unroll
-                    for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
-                }
-                if (j == t0 + q) out = p;
+            for (int i = 0; i < UPL; ++i) {
+                const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
+                bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
             }
         }
-        // entry l = t*G+g was kept by lane g*LPN+t
+    };
+    auto consume = [&](const Ent &x, int t0, int steps, const T (&bf)[NB][UPL], float &out) {
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            if (t0 + q >= steps) break;               // wave-uniform
+            const int src = ((t0 + q) * G + g) & (WAVE - 1);
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                const float d = U::dot(a.u[i], bf[q][i], p);
+                p = C::unit_on(j, i, KU) ? d : p;
+            }
+            // a step past the end of the row works on a clamped position: it must leave the
+            // output row alone whatever that position's B row holds (0 * inf is not 0)
+            const bool live = __shfl((int)x.valid, src, WAVE) != 0;
+            p = group_sum<LPN>(p) * __shfl(x.s, src, WAVE);   // every lane takes part in the lane exchange
+            p = live ? p : 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                float next[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e) next[e] = acc[i][e];
+                U::axpy(p, bf[q][i], next);
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
+            }
+            if (j == t0 + q) out = p;
+        }
+    };
+    auto steps_of = [&](int base) {
+        const int count = end - base < WAVE ? end - base : WAVE;
+        const int st = (count + G - 1) / G;
+        return st < LPN ? st : LPN;
+    };
+    // entry l = t*G+g was kept by lane g*LPN+t
+    auto store_p = [&](const Ent &x, float out) {
         const float res = __shfl(out, (lane % G) * LPN + lane / G, WAVE);
-        if (valid) P[n] = res;
+        if (x.valid) P[x.n] = res;
+    };
+    // Batches of NB steps, LPN / NB of them per chunk of 64 entries: the gathers of the next batch (of
+    // the next chunk after a chunk's last) and the indices of the chunk after the next are in flight
+    // while a batch is multiplied, one round trip per batch instead of one per batch and one per chunk.
+    constexpr int BPC = LPN / NB;
+    static_assert(LPN % NB == 0, "whole batches per chunk");
+    // (Rows of more than one unit per lane keep one batch in flight: the second buffer costs them a
+    // third of their wavefronts per SIMD, 171 against 153 us on banded rows of 256 bytes.)
+    constexpr bool AHEAD = UPL == 1;
+    Ent cur = entry(start);
+    T bcur[NB][UPL];
+    if constexpr (AHEAD) gather(cur, 0, bcur);
+    Ent nxt = entry(start + WAVE);
+    for (int base = start; base < end; base += WAVE) {
+        const int steps = steps_of(base);
+        const bool more = base + WAVE < end;
+        const Ent after = entry(base + 2 * WAVE);
+        float out = 0.f;
+#pragma unroll
+        for (int bq = 0; bq < BPC; ++bq) {
+            const int t0 = bq * NB;
+            if (t0 >= steps) break;                           // wave-uniform
+            if constexpr (AHEAD) {
+                T bnxt[NB][UPL];
+                if (bq + 1 < BPC && t0 + NB < steps) gather(cur, t0 + NB, bnxt);
+                else if (more) gather(nxt, 0, bnxt);
+                consume(cur, t0, steps, bcur, out);
+#pragma unroll
+                for (int q = 0; q < NB; ++q)
+#pragma unroll
+                    for (int i = 0; i < UPL; ++i) bcur[q][i] = bnxt[q][i];
+            } else {
+                gather(cur, t0, bcur);
+                consume(cur, t0, steps, bcur, out);
+            }
+        }
+        store_p(cur, out);
+        cur = nxt;
+        nxt = after;
     }
     // add the partial output rows of the G groups: lanes with the same j
 #pragma unroll
@@ -142,8 +189,9 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm(const void *__restrict__ A, c
 // S value of entry t0+j, so LPN entries of each row are gathered back to back; the
 // P value of entry t0+j ends up in lane j, and the output row needs no reduction
 // across groups.  Longer rows are left to k_fusedmm and the rows of 8-row panels
-// (panel_owner[row] == 2, when the array is given) to the panel kernel (they count as
-// empty here); every other row, empty ones included, gets its output row written.
+// (panel_owner[row] == 2, when the array is given) to the panel kernel: those rows count
+// as empty here and get a row of zeros, which the kernels launched after this one add to.
+// Every row below M gets its output row written, so O needs no clearing before the launch.
 template <class L>
 __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__ A, const void *__restrict__ B, int KU,
                                                         const int32_t *__restrict__ rowptr,
@@ -186,57 +234,96 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
     for (int i = 0; i < UPL; ++i)
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[i][e] = 0.f;
-    for (int t0 = 0; t0 < longest; t0 += LPN) {
+    struct Ent { int at, c; float s; bool has; };
+    auto entry = [&](int t0) {                        // entry t0 + j of this group's row
+        Ent x;
         const int e = t0 + j;
-        const bool has = e < len;
-        const int at = has ? rs + e : (len > 0 ? rs + len - 1 : 0);   // a valid position in every lane
-        const int c = col[at];
-        const float s = has ? sval[at] : 0.f;
-        const Off_t boff = (Off_t)c * rb;
-        const int steps = longest - t0 < LPN ? longest - t0 : LPN;
-        float out = 0.f;
-        for (int q0 = 0; q0 < steps; q0 += NB) {
-            T bf[NB][UPL];
+        x.has = e < len;
+        x.at = x.has ? rs + e : (len > 0 ? rs + len - 1 : 0);   // a valid position in every lane
+        x.c = col[x.at];
+        x.s = x.has ? sval[x.at] : 0.f;
+        return x;
+    };
+    auto gather = [&](const Ent &x, int q0, T (&bf)[NB][UPL]) {
+        const Off_t boff = (Off_t)x.c * rb;
 #pragma unroll
-            for (int q = 0; q < NB; ++q) {
-                const int src = g * LPN + ((q0 + q) & (LPN - 1));
-                const Off_t bo = shfl_off<Off_t>(boff, src);
+        for (int q = 0; q < NB; ++q) {
+            const int src = g * LPN + ((q0 + q) & (LPN - 1));
+            const Off_t bo = shfl_off<Off_t>(boff, src);
 #pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
-                    bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
-                }
-            }
-#pragma unroll
-            for (int q = 0; q < NB; ++q) {
-                if (q0 + q >= steps) break;               // wave-uniform
-                const int src = g * LPN + ((q0 + q) & (LPN - 1));
-                float p = 0.f;
-#pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    const float d = U::dot(a.u[i], bf[q][i], p);
-                    p = C::unit_on(j, i, KU) ? d : p;
-                }
-                // a step past the end of the row works on a clamped position: it must leave the
-                // output row alone whatever that position's B row holds (0 * inf is not 0)
-                const bool live = __shfl((int)has, src, WAVE) != 0;
-                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);     // every lane takes part in the lane exchange
-                p = live ? p : 0.f;
-#pragma unroll
-                for (int i = 0; i < UPL; ++i) {
-                    float next[E];
-#pragma unroll
-                    for (int e = 0; e < E; ++e) next[e] = acc[i][e];
-                    U::axpy(p, bf[q][i], next);
-#pragma unroll
-                    for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
-                }
-                if (j == q0 + q) out = p;
+            for (int i = 0; i < UPL; ++i) {
+                const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
+                bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
             }
         }
-        if (has) P[at] = out;
+    };
+    auto consume = [&](const Ent &x, int q0, int steps, const T (&bf)[NB][UPL], float &out) {
+#pragma unroll
+        for (int q = 0; q < NB; ++q) {
+            if (q0 + q >= steps) break;               // wave-uniform
+            const int src = g * LPN + ((q0 + q) & (LPN - 1));
+            float p = 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                const float d = U::dot(a.u[i], bf[q][i], p);
+                p = C::unit_on(j, i, KU) ? d : p;
+            }
+            // a step past the end of the row works on a clamped position: it must leave the
+            // output row alone whatever that position's B row holds (0 * inf is not 0)
+            const bool live = __shfl((int)x.has, src, WAVE) != 0;
+            p = group_sum<LPN>(p) * __shfl(x.s, src, WAVE);   // every lane takes part in the lane exchange
+            p = live ? p : 0.f;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                float next[E];
+#pragma unroll
+                for (int e = 0; e < E; ++e) next[e] = acc[i][e];
+                U::axpy(p, bf[q][i], next);
+#pragma unroll
+                for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
+            }
+            if (j == q0 + q) out = p;
+        }
+    };
+    // Batches of NB steps, LPN / NB of them per LPN entries of a row: the gathers of the next batch and
+    // the indices of the entries after the next LPN are in flight while a batch is multiplied.
+    constexpr int BPC = LPN / NB;
+    static_assert(LPN % NB == 0, "whole batches per LPN entries");
+    constexpr bool AHEAD = UPL <= 2;                 // (rows of more units per lane: measured the same either way)
+    Ent cur = entry(0);
+    T bcur[NB][UPL];
+    if constexpr (AHEAD) {
+        if (longest > 0) gather(cur, 0, bcur);                // wave-uniform
     }
-    if (mine) {
+    Ent nxt = entry(LPN);
+    for (int t0 = 0; t0 < longest; t0 += LPN) {
+        const int steps = longest - t0 < LPN ? longest - t0 : LPN;
+        const bool more = t0 + LPN < longest;
+        const Ent after = entry(t0 + 2 * LPN);
+        float out = 0.f;
+#pragma unroll
+        for (int bq = 0; bq < BPC; ++bq) {
+            const int q0 = bq * NB;
+            if (q0 >= steps) break;                           // wave-uniform
+            if constexpr (AHEAD) {
+                T bnxt[NB][UPL];
+                if (bq + 1 < BPC && q0 + NB < steps) gather(cur, q0 + NB, bnxt);
+                else if (more) gather(nxt, 0, bnxt);
+                consume(cur, q0, steps, bcur, out);
+#pragma unroll
+                for (int q = 0; q < NB; ++q)
+#pragma unroll
+                    for (int i = 0; i < UPL; ++i) bcur[q][i] = bnxt[q][i];
+            } else {
+                gather(cur, q0, bcur);
+                consume(cur, q0, steps, bcur, out);
+            }
+        }
+        if (cur.has) P[cur.at] = out;
+        cur = nxt;
+        nxt = after;
+    }
+    if (row < M) {                                    // (the accumulators of a row left to other kernels are zero)
         float *orow = O + row * KU * E;
 #pragma unroll
         for (int i = 0; i < UPL; ++i) {

@@ -1682,13 +1682,19 @@ int sddmm_run_fused(sddmm_ctx *c) {
         c->o_cap = o_bytes;
     }
     HIP_TRY(c, hipEventRecord(c->ev0, c->stream));
-    if (o_bytes) HIP_TRY(c, hipMemsetAsync(c->dO, 0, o_bytes, c->stream));
+    // (when the panels own every row that has entries, O is complete after a memset and the panel kernel;
+    // otherwise the kernel of the short rows, first in the stream, writes every row of O below sM, zeros
+    // for the rows that the kernels after it add to, and only the rows of A beyond S are cleared here)
+    const bool others = c->sM > 0 && c->nnz > 0 && (!panels || c->n_tiles > 0 || c->rows_short > 0 || c->n_items > 0);
+    if (o_bytes) {
+        const size_t written = others ? (size_t)c->sM * (size_t)c->K * sizeof(float) : 0;
+        if (written < o_bytes) HIP_TRY(c, hipMemsetAsync((char *)c->dO + written, 0, o_bytes - written, c->stream));
+    }
     int launches = 0;
+    bool rows_written = false;
     if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);
-            // (when the panels own every row that has entries, O is complete after the memset and the panel kernel)
-            const bool others = !panels || c->n_tiles > 0 || c->rows_short > 0 || c->n_items > 0;
             if (!others) return;
             if constexpr (!LT::LONG && LT::LPN <= 8 && LT::U::ELEMS > 1 && LT::UPL * LT::U::ELEMS <= 32) {
                 const int64_t rows_per_wave = WAVE / LT::LPN;
@@ -1698,6 +1704,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
                                    (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
                                    c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks, panel_owner);
                 ++launches;
+                rows_written = true;
                 if (c->n_fused_items > 0) {
                     const int64_t nblocks = (c->n_fused_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
                     SDDMM_LAUNCH(c, (k_fusedmm<LT>), xcd_grid(nblocks), BLOCK,
@@ -1708,6 +1715,7 @@ int sddmm_run_fused(sddmm_ctx *c) {
                 }
             }
         });
+        if (others && !rows_written) return fail(c, SDDMM_ERR_UNSUPPORTED, "internal: no fused kernel for this row layout");
         if (panels) {
             if (c->dtype == SDDMM_F32) {
                 if (c->K == 32) launch_panel_fused_t<DT_F32, 2>(c);

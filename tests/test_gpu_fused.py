@@ -176,6 +176,37 @@ def test_fused_non_finite_rows_of_b_stay_in_their_own_entries(engine_factory):
     e.close()
 
 
+def test_fused_output_rows_keep_nothing_of_an_earlier_call(engine_factory):
+    """O is written, not cleared and added to, for the rows the short-row kernel owns: a second call on
+    the same context with fewer rows in S, other rows long and other rows empty must not show anything
+    of the first call's output, and the rows of A beyond S's rows come back as zeros."""
+    rng = np.random.default_rng(611)
+    MA, N, K = 96, 700, 32
+    A = rng.uniform(-1, 1, (MA, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    e = engine_factory()
+    e.set_dense(A, B)
+
+    def pattern(M, lens):
+        rows = [np.sort(rng.choice(N, int(n), replace=False)) for n in lens]
+        rowptr = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int32)
+        col = np.concatenate(rows).astype(np.int32) if rowptr[-1] else np.zeros(0, np.int32)
+        return rowptr, col, rng.uniform(-1, 1, len(col)).astype(f32)
+
+    lens1 = rng.choice([0, 3, 20, 64, 65, 300, 650], MA)
+    rowptr, col, val = pattern(MA, lens1)
+    e.set_csr(MA, N, rowptr, col, val)
+    _check(e, rowptr, col, val, A, B, "first call")
+    M2 = 60
+    lens2 = np.where(lens1[:M2] > 64, 0, 500)             # long rows become empty, the others long
+    lens2[::7] = 5
+    rowptr, col, val = pattern(M2, lens2)
+    e.set_csr(M2, N, rowptr, col, val)
+    got = _check(e, rowptr, col, val, A[:M2], B, "second call, fewer rows")
+    assert got.shape[0] == MA and not got[M2:].any()
+    e.close()
+
+
 def _panel_pattern(rng, N, panel_lens, loose_lens):
     """8-row panels (one column list per panel) with loose rows in between, in groups of 8 so
     that the panels stay 8-aligned."""
