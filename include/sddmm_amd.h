@@ -227,11 +227,12 @@ int sddmm_launch_noalloc(int M, int N, int K, int64_t nnz, const float *dA, cons
  * Rows cut into several work items (longer than 2048 entries; longer than 256 where a
  * matrix of rows of up to 128 bytes has only a few thousand such rows) are accumulated
  * with atomic adds, so their last bits may differ from run to run.
- * fp32 operands with K = 32, 64 or 128: the rows that the current plan (SDDMM_AUTO is planned
- * if there is none) runs as 8-row panels take a matrix-core kernel that shares every
- * gathered B row between the 8 rows and between both products; panels whose column list
- * is cut into several work items (more than 512 columns) are accumulated with atomic adds
- * as above.  The other rows take the gather kernels. */
+ * K = 32, 64 or 128 (fp32, bf16 or fp16 operands): the rows that the current plan (SDDMM_AUTO
+ * is planned if there is none) runs as 8-row panels take a matrix-core kernel that shares
+ * every gathered B row between the 8 rows and between both products; the output rows of a
+ * panel are accumulated with atomic adds as above.  The other rows take the gather kernels.
+ * In either kernel a B row is read only for entries that are stored: a non-finite value in B
+ * reaches the output rows that have an entry in its column and no others. */
 int sddmm_run_fused(sddmm_ctx *ctx);
 int sddmm_get_fused(sddmm_ctx *ctx, float *O);                    /* M*K floats to the host */
 int sddmm_get_fused_device(sddmm_ctx *ctx, const float **dO);     /* valid until the next set_* / destroy */
