@@ -63,14 +63,22 @@ def test_full_size(engine_factory, name, K, other):
     e.close()
 
 
-@pytest.mark.parametrize("name,K", [("fem_banded", 32), ("fem_banded", 128), ("mixed_density", 64)])
-def test_fused_full_size(engine_factory, name, K):
-    """SDDMM followed by SpMM at the benchmark's sizes: the panel kernel (fem_banded) and the
-    gather kernels (mixed_density) against the oracle, and the row sums of O against float64."""
+@pytest.mark.parametrize("name,K,dtype", [("fem_banded", 32, capi.F32), ("fem_banded", 128, capi.F32),
+                                          ("mixed_density", 64, capi.F32), ("fem_banded", 64, capi.BF16),
+                                          ("power_law", 32, capi.F32)])
+def test_fused_full_size(engine_factory, name, K, dtype):
+    """SDDMM followed by SpMM at the benchmark's sizes: the panel kernel (fem_banded, fp32 and bf16
+    operands) and the gather kernels (mixed_density, power_law) against the oracle on the operands as
+    stored, and the row sums of O against float64."""
     w = W.make(name, "full", K=K)
     print("fused full size", name, K, "nnz", w.nnz, flush=True)
     e = engine_factory()
-    e.set_dense(w.A, w.B)
+    if dtype == capi.BF16:
+        Ab, Bb = capi.to_bf16(w.A).reshape(w.A.shape), capi.to_bf16(w.B).reshape(w.B.shape)
+        w.A, w.B = capi.from_bf16(Ab).reshape(w.A.shape), capi.from_bf16(Bb).reshape(w.B.shape)
+        e.set_dense(Ab, Bb, capi.BF16)
+    else:
+        e.set_dense(w.A, w.B)
     e.set_csr(w.M, w.N, w.rowptr, w.col, w.sval)
     e.plan(capi.AUTO)
     got_o = e.run_fused()
