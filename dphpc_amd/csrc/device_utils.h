@@ -46,6 +46,14 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 // index of the wavefront inside its workgroup, as a scalar
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
+// LDS that only one wavefront touches: its LDS operations execute in program order, so a
+// write followed by a read of another lane's slot needs no workgroup barrier, only that the
+// compiler keeps the order.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 // Workgroups are handed to the 8 XCDs round-robin by id.  Give every XCD one
 // contiguous eighth of the logical work so that neighbouring row panels (which
 // touch neighbouring B rows) share an L2.  Returns the logical index, or -1 for

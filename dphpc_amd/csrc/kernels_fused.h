@@ -337,4 +337,179 @@ __global__ __launch_bounds__(BLOCK) void k_fusedmm_rows(const void *__restrict__
     }
 }
 
+// The same rows as k_fusedmm_rows when their lengths differ a lot (a power-law graph: most
+// rows hold one to three entries, a few dozens): there a lane group that waits for the longest
+// of a wavefront's 64/LPN rows idles four steps out of five.  Here a wavefront takes 64
+// consecutive rows, numbers their entries across the rows (prefix sum of the lengths, kept in
+// LDS with the rows' CSR positions) and deals whole rows out to its lane groups so that every
+// group gets about an equal share of the entries.  A group walks its entries LPN at a time: lane
+// j finds the row of its entry by bisection over the prefix sums, loads column index and S
+// value; step q then takes entry q with all lanes of the group, gathers the entry's A row with
+// its B row (the rows change inside a group, as in the flat kernel), and the group's partial
+// output row is written whenever the row changes.  Rows without entries of their own (empty,
+// left to other kernels) get zeros, as in k_fusedmm_rows.
+template <class L>
+__global__ __launch_bounds__(BLOCK) void k_fusedmm_rows_balanced(const void *__restrict__ A, const void *__restrict__ B,
+                                                                 int KU, const int32_t *__restrict__ rowptr,
+                                                                 const int32_t *__restrict__ col,
+                                                                 const float *__restrict__ sval, float *__restrict__ P,
+                                                                 float *__restrict__ O, int M, int max_len,
+                                                                 int64_t nblocks,
+                                                                 const unsigned char *__restrict__ panel_owner) {
+    using U = typename L::U;
+    using T = typename U::T;
+    constexpr int E = U::ELEMS;
+    using C = Chunk<U, L::LPN, L::UPL, L::FULLK, false, L::WIDE>;
+    using Off_t = typename C::O;
+    constexpr int LPN = L::LPN, UPL = L::UPL, G = WAVE / LPN;
+    constexpr int NB = C::BIG > 4 ? 4 : C::BIG;       // A and B rows of a batch of steps in flight together
+    __shared__ int pre_all[WAVES_PER_BLOCK][WAVE], pos_all[WAVES_PER_BLOCK][WAVE];
+    const int64_t blk = xcd_remap(blockIdx.x, nblocks);
+    if (blk < 0) return;
+    const int64_t r0 = (blk * WAVES_PER_BLOCK + wave_in_block()) * WAVE;
+    if (r0 >= M) return;
+    const int lane = lane_id();
+    const int g = lane / LPN, j = lane & (LPN - 1);
+    int *pre = pre_all[wave_in_block()], *pos = pos_all[wave_in_block()];
+    // lane l: row r0 + l
+    const bool inside = r0 + lane < M;
+    int rs = 0, len = 0;
+    if (inside) {
+        rs = rowptr[r0 + lane];
+        len = rowptr[r0 + lane + 1] - rs;
+        if (len > max_len || (panel_owner && panel_owner[r0 + lane] == 2)) len = 0;
+    }
+    int incl = len;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const int up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
+    }
+    const int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
+    pre[lane] = incl - len;
+    pos[lane] = rs;
+    wave_lds_order();
+    // whole rows per group: group gg starts at the first row whose prefix reaches gg/G of the entries
+    int b_lo = 0, b_hi = WAVE;
+#pragma unroll
+    for (int gg = 1; gg < G; ++gg) {
+        const int target = (int)((int64_t)gg * total / G);
+        const int first = __popcll(__ballot(incl - len < target));
+        if (g == gg) b_lo = first;
+        if (g + 1 == gg) b_hi = first;
+    }
+    const int v_lo = b_lo < WAVE ? pre[b_lo] : total, v_hi = b_hi < WAVE ? pre[b_hi] : total;
+    int longest = v_hi - v_lo;
+#pragma unroll
+    for (int o = LPN; o < WAVE; o <<= 1) {
+        const int other = __shfl_xor(longest, o, WAVE);
+        longest = other > longest ? other : longest;
+    }
+    longest = __builtin_amdgcn_readfirstlane(longest);
+    const Off_t rb = (Off_t)KU * (Off_t)sizeof(T);
+    // rows with nothing of their own: zeros (lane group g takes rows g, g + G, ..)
+    {
+        const unsigned long long empty = __ballot(inside && len == 0);
+#pragma unroll
+        for (int k = 0; k < WAVE / G; ++k) {
+            const int rr = k * G + g;
+            if (!((empty >> rr) & 1ull)) continue;
+            float *orow = O + (r0 + rr) * (int64_t)KU * E;
+#pragma unroll
+            for (int i = 0; i < UPL; ++i) {
+                const int u = j + i * LPN;
+                if (!C::unit_on(j, i, KU)) continue;
+#pragma unroll
+                for (int e = 0; e < E; e += 4)
+                    *reinterpret_cast<float4 *>(orow + E * u + e) = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+    float acc[UPL][E];
+#pragma unroll
+    for (int i = 0; i < UPL; ++i)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[i][e] = 0.f;
+    int cur_row = -1;                                 // the row the group's partial sums belong to (the same in its lanes)
+    auto flush = [&](bool on) {
+        if (!on) return;
+        float *orow = O + (r0 + cur_row) * (int64_t)KU * E;
+#pragma unroll
+        for (int i = 0; i < UPL; ++i) {
+            const int u = j + i * LPN;
+            if (!C::unit_on(j, i, KU)) continue;
+#pragma unroll
+            for (int e = 0; e < E; e += 4)
+                *reinterpret_cast<float4 *>(orow + E * u + e) =
+                    make_float4(acc[i][e], acc[i][e + 1], acc[i][e + 2], acc[i][e + 3]);
+        }
+    };
+    for (int t0 = 0; t0 < longest; t0 += LPN) {
+        const int v = v_lo + t0 + j;
+        const bool has = v < v_hi;
+        // the row of entry v: the last row whose prefix does not exceed v (rows without entries
+        // share their prefix with the row after them and are never the last such row)
+        const int vv = has ? v : (v_hi > v_lo ? v_hi - 1 : 0);
+        int lo = 0, hi = WAVE;
+#pragma unroll
+        for (int it = 0; it < 6; ++it) {
+            const int mid = (lo + hi) >> 1;
+            if (pre[mid] <= vv) lo = mid; else hi = mid;
+        }
+        const int row = v_hi > v_lo ? lo : 0;                            // (a group without entries: row 0, position 0)
+        const int at = v_hi > v_lo ? pos[row] + (vv - pre[row]) : 0;      // a valid position in every lane
+        const int c = col[at];
+        const float s = has ? sval[at] : 0.f;
+        const Off_t boff = (Off_t)c * rb, aoff = (Off_t)(r0 + row) * rb;
+        const int steps = longest - t0 < LPN ? longest - t0 : LPN;
+        float out = 0.f;
+        for (int q0 = 0; q0 < steps; q0 += NB) {
+            T bf[NB][UPL], af[NB][UPL];
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const int src = g * LPN + ((q0 + q) & (LPN - 1));
+                const Off_t bo = shfl_off<Off_t>(boff, src), ao = shfl_off<Off_t>(aoff, src);
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const int u = C::unit_on(j, i, KU) ? j + i * LPN : 0;
+                    bf[q][i] = load_at<T, Off_t>(B, bo + (Off_t)(u * (int)sizeof(T)));
+                    af[q][i] = load_at<T, Off_t>(A, ao + (Off_t)(u * (int)sizeof(T)));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                if (q0 + q >= steps) break;               // wave-uniform
+                const int src = g * LPN + ((q0 + q) & (LPN - 1));
+                const bool live = __shfl((int)has, src, WAVE) != 0;
+                const int row_q = __shfl(row, src, WAVE);
+                const bool change = live && row_q != cur_row;
+                flush(change && cur_row >= 0);
+                cur_row = change ? row_q : cur_row;
+                float p = 0.f;
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    const float d = U::dot(af[q][i], bf[q][i], p);
+                    p = C::unit_on(j, i, KU) ? d : p;
+                }
+                // a step past the end of the group's entries works on a clamped position: it must leave
+                // the output row alone whatever that position's B row holds (0 * inf is not 0)
+                p = group_sum<LPN>(p) * __shfl(s, src, WAVE);     // every lane takes part in the lane exchange
+                p = live ? p : 0.f;
+#pragma unroll
+                for (int i = 0; i < UPL; ++i) {
+                    float next[E];
+#pragma unroll
+                    for (int e = 0; e < E; ++e) next[e] = change ? 0.f : acc[i][e];
+                    U::axpy(p, bf[q][i], next);
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[i][e] = live ? next[e] : acc[i][e];
+                }
+                if (j == q0 + q) out = p;
+            }
+        }
+        if (has) P[at] = out;
+    }
+    flush(cur_row >= 0);
+}
+
 }  // namespace sddmm

@@ -158,11 +158,6 @@ constexpr int STRIP_BM_WORDS = 1024;          // 32768 tile columns: a span of 5
 constexpr int STRIP_UNROLL = 4;               // loads of 256 entries per batch, two batches in flight
 constexpr int STRIPS_PER_BLOCK = 4;
 
-__device__ __forceinline__ void wave_lds_order() {
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-}
-
 __device__ __forceinline__ int wave_sum_i32(int v) {
     for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
     return v;

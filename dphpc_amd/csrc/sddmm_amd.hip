@@ -124,6 +124,7 @@ struct sddmm_ctx {
     int64_t n_fused_items = 0, fused_items_cap = 0;
     bool fused_items_valid = false;
     bool fused_items_panels = false; // the fused items leave out the rows that the panel kernel owns
+    double fused_short_avg = 0.0;    // entries per non-empty row of at most FUSED_ROW_MAX entries (panel rows apart)
     float *dO = nullptr;
     size_t o_cap = 0;
     bool have_fused = false;
@@ -1622,6 +1623,7 @@ static int plan_fused_items(sddmm_ctx *c, const unsigned char *panel_owner) {
         // times the long segments stay: there the atomic adds cost more than they return.
         const PlanCounters first = summarize(tmp);
         const int64_t item_entries = (int64_t)(first.nnz_medium + first.nnz_long);
+        c->fused_short_avg = first.rows_short ? (double)first.nnz_short / (double)first.rows_short : 0.0;
         // (rows of up to 128 bytes; at 256 bytes it changes nothing, at 1 KiB the adds of 256 floats per piece lose 4 %)
         if ((int64_t)tmp.n_items > 0 && (int64_t)tmp.n_items < 4096 && !getenv("SDDMM_FUSED_SEG") &&
             (size_t)c->K * elem_size(c->dtype) <= 128) {
@@ -1692,6 +1694,13 @@ int sddmm_run_fused(sddmm_ctx *c) {
     }
     int launches = 0;
     bool rows_written = false;
+    // Rows of fewer entries than a lane group takes per step, on average (a power-law graph: 3.5): one row per
+    // lane group would idle most of its steps (20 % of them useful there), so the wavefronts deal whole
+    // rows out to their groups by entry count instead (1 088 -> 881 us on that shape; with longer rows
+    // the extra gathers of the A rows and the longer walks cost more than the idle steps: 33 -> 65 us on
+    // the mixed-density shape, 12.5 entries per short row).
+    const int balanced_env = env_int("SDDMM_FUSED_BALANCED", -1);
+    const bool balanced = balanced_env >= 0 ? balanced_env != 0 : (c->fused_short_avg > 0.0 && c->fused_short_avg < 8.0);
     if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);
@@ -1700,9 +1709,17 @@ int sddmm_run_fused(sddmm_ctx *c) {
                 const int64_t rows_per_wave = WAVE / LT::LPN;
                 const int64_t waves = ((int64_t)c->sM + rows_per_wave - 1) / rows_per_wave;
                 const int64_t rblocks = (waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
-                SDDMM_LAUNCH(c, (k_fusedmm_rows<LT>), xcd_grid(rblocks), BLOCK,
-                                   (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
-                                   c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks, panel_owner);
+                if (balanced) {
+                    const int64_t bwaves = ((int64_t)c->sM + WAVE - 1) / WAVE;
+                    const int64_t bblocks = (bwaves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+                    SDDMM_LAUNCH(c, (k_fusedmm_rows_balanced<LT>), xcd_grid(bblocks), BLOCK,
+                                       (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
+                                       c->dP, c->dO, c->sM, FUSED_ROW_MAX, bblocks, panel_owner);
+                } else {
+                    SDDMM_LAUNCH(c, (k_fusedmm_rows<LT>), xcd_grid(rblocks), BLOCK,
+                                       (const void *)c->dA, (const void *)c->dB, s.KU, c->d_rowptr, c->d_col, c->d_sval,
+                                       c->dP, c->dO, c->sM, FUSED_ROW_MAX, rblocks, panel_owner);
+                }
                 ++launches;
                 rows_written = true;
                 if (c->n_fused_items > 0) {

@@ -207,6 +207,52 @@ def test_fused_output_rows_keep_nothing_of_an_earlier_call(engine_factory):
     e.close()
 
 
+@pytest.mark.parametrize("K", [8, 32, 64, 128])
+@pytest.mark.parametrize("forced", [False, True])
+def test_fused_rows_of_very_different_lengths(engine_factory, monkeypatch, K, forced):
+    """A power-law-like pattern (most rows one to three entries, many empty, a few dozens, some beyond
+    64): the short rows average fewer than 8 entries, so the wavefronts deal whole rows out to their
+    lane groups by entry count (forced: the same kernel on rows of 20 to 40 entries too).  A row count
+    that is no multiple of 64, rows of A beyond S's rows, an infinity in a B row that one short row has."""
+    if forced:
+        monkeypatch.setenv("SDDMM_FUSED_BALANCED", "1")
+    rng = np.random.default_rng(7300 + K + forced)
+    M, MA, N = 64 * 37 + 29, 64 * 37 + 40, 5000
+    lens = rng.choice([0, 0, 1, 1, 1, 2, 2, 3, 5, 9, 30, 64, 65, 200] if not forced else [0, 20, 25, 33, 40, 64, 65], M)
+    lens[:64] = 0                                         # a wavefront without entries
+    lens[64:128] = 1
+    lens[200] = 64
+    rows = [np.sort(rng.choice(N - 1, int(n), replace=False)) for n in lens]
+    rows[130] = np.array([5, N - 1])
+    lens[130] = 2
+    rowptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col = np.concatenate(rows).astype(np.int32)
+    val = rng.uniform(-1, 1, len(col)).astype(f32)
+    A = rng.uniform(-1, 1, (MA, K)).astype(f32)
+    B = rng.uniform(-1, 1, (N, K)).astype(f32)
+    e = engine_factory()
+    e.set_dense(A, B)
+    e.set_csr(M, N, rowptr, col, val)
+    e.plan(capi.AUTO)
+    got = _check(e, rowptr, col, val, A[:M], B, "rows of very different lengths K=%d" % K)
+    assert got.shape[0] == MA and not got[M:].any()
+    B2 = B.copy()
+    B2[N - 1, K // 2] = np.inf
+    e.set_dense(A, B2)
+    e.set_csr(M, N, rowptr, col, val)
+    e.plan(capi.AUTO)
+    got = e.run_fused()
+    bad = ~np.isfinite(got).all(axis=1)
+    assert bad[130] and bad.sum() == 1
+    with np.errstate(all="ignore"):
+        _, ref_o = O.fusedmm_csr(rowptr, col, val, A[:M], B2)
+        _, mag_o = O.fusedmm_csr_f64(rowptr, col, val, A[:M], B2)
+    keep = ~bad[:M]
+    ok, worst, i = O.check_values(got[:M][keep].ravel(), ref_o[keep].ravel(), mag=mag_o[keep].ravel())
+    assert ok, (K, forced, i, worst)
+    e.close()
+
+
 def _panel_pattern(rng, N, panel_lens, loose_lens):
     """8-row panels (one column list per panel) with loose rows in between, in groups of 8 so
     that the panels stay 8-aligned."""
