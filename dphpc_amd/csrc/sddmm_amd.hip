@@ -1694,13 +1694,15 @@ int sddmm_run_fused(sddmm_ctx *c) {
     }
     int launches = 0;
     bool rows_written = false;
-    // Rows of fewer entries than a lane group takes per step, on average (a power-law graph: 3.5): one row per
-    // lane group would idle most of its steps (20 % of them useful there), so the wavefronts deal whole
-    // rows out to their groups by entry count instead (1 088 -> 881 us on that shape; with longer rows
-    // the extra gathers of the A rows and the longer walks cost more than the idle steps: 33 -> 65 us on
-    // the mixed-density shape, 12.5 entries per short row).
+    // Short rows of fewer entries, on average, than half of what a lane group takes per step (a power-law
+    // graph: 3.5 against 8 lanes per entry at 128-byte rows): one row per lane group would idle most of its
+    // steps (20 % of them useful there), so the wavefronts deal whole rows out to their groups by entry
+    // count instead (576 -> 369 us for those rows).  With longer rows, or 4 lanes per entry, the extra
+    // gathers of the A rows and the longer walks cost more than the idle steps (mixed-density shape, 12.5
+    // entries per short row: 33 -> 65 us; power-law with 64-byte rows: 396 -> 432 us).
     const int balanced_env = env_int("SDDMM_FUSED_BALANCED", -1);
-    const bool balanced = balanced_env >= 0 ? balanced_env != 0 : (c->fused_short_avg > 0.0 && c->fused_short_avg < 8.0);
+    const bool balanced = balanced_env >= 0 ? balanced_env != 0
+                                            : (c->fused_short_avg > 0.0 && 2.0 * c->fused_short_avg < (double)s.LPN);
     if (c->sM > 0 && c->nnz > 0) {
         with_layout(s, [&](auto L) {
             using LT = decltype(L);

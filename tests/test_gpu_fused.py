@@ -211,14 +211,15 @@ def test_fused_output_rows_keep_nothing_of_an_earlier_call(engine_factory):
 @pytest.mark.parametrize("forced", [False, True])
 def test_fused_rows_of_very_different_lengths(engine_factory, monkeypatch, K, forced):
     """A power-law-like pattern (most rows one to three entries, many empty, a few dozens, some beyond
-    64): the short rows average fewer than 8 entries, so the wavefronts deal whole rows out to their
-    lane groups by entry count (forced: the same kernel on rows of 20 to 40 entries too).  A row count
+    64): the short rows average 3.2 entries, fewer than half the 8 lanes of an entry at K >= 32, so the
+    wavefronts deal whole rows out to their lane groups by entry count (forced: that kernel whatever K
+    and on rows of 20 to 40 entries too).  A row count
     that is no multiple of 64, rows of A beyond S's rows, an infinity in a B row that one short row has."""
     if forced:
         monkeypatch.setenv("SDDMM_FUSED_BALANCED", "1")
     rng = np.random.default_rng(7300 + K + forced)
     M, MA, N = 64 * 37 + 29, 64 * 37 + 40, 5000
-    lens = rng.choice([0, 0, 1, 1, 1, 2, 2, 3, 5, 9, 30, 64, 65, 200] if not forced else [0, 20, 25, 33, 40, 64, 65], M)
+    lens = rng.choice([0, 0, 1, 1, 1, 1, 1, 1, 2, 2, 2, 3, 3, 20, 65, 200] if not forced else [0, 20, 25, 33, 40, 64, 65], M)
     lens[:64] = 0                                         # a wavefront without entries
     lens[64:128] = 1
     lens[200] = 64
