@@ -557,6 +557,30 @@ __global__ __launch_bounds__(256) void k_gather_candidates(const int32_t *__rest
     }
 }
 
+// The candidate keys in increasing order when there are at most RANK_SORT_MAX of them: every
+// workgroup holds all keys in LDS and finds the ranks of 8 of them, 32 threads per key (keys are
+// distinct, one per row, so the ranks are a permutation).  One short launch instead of the
+// passes of a radix sort over 64-bit keys.
+#ifndef SDDMM_RANK_SORT_SPLIT
+#define SDDMM_RANK_SORT_SPLIT 32
+#endif
+constexpr int RANK_SORT_MAX = 8192, RANK_SORT_BLOCK = 256, RANK_SORT_SPLIT = SDDMM_RANK_SORT_SPLIT;
+__global__ __launch_bounds__(RANK_SORT_BLOCK) void k_rank_sort(const unsigned long long *__restrict__ in,
+                                                               unsigned long long *__restrict__ out, int n) {
+    __shared__ unsigned long long v[RANK_SORT_MAX];
+    for (int i = (int)threadIdx.x; i < n; i += RANK_SORT_BLOCK) v[i] = in[i];
+    __syncthreads();
+    const int idx = (int)blockIdx.x * (RANK_SORT_BLOCK / RANK_SORT_SPLIT) + (int)(threadIdx.x / RANK_SORT_SPLIT);
+    const int part = (int)(threadIdx.x % RANK_SORT_SPLIT);
+    const unsigned long long mine = v[idx < n ? idx : n - 1];
+    int below = 0;
+#pragma unroll 8
+    for (int i = part; i < n; i += RANK_SORT_SPLIT) below += v[i] < mine ? 1 : 0;
+#pragma unroll
+    for (int o = 1; o < RANK_SORT_SPLIT; o <<= 1) below += __shfl_xor(below, o, WAVE);
+    if (part == 0 && idx < n) out[below] = mine;
+}
+
 // Gathered strips come in PAIRS: 32 consecutive candidates of the sorted order, the first 16
 // as strip 2p, the rest as strip 2p+1, with ONE list of tile columns -- every tile column that
 // any of the 32 rows touches -- so that the two strips have the same descriptors in the same

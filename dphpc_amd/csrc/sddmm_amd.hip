@@ -733,17 +733,25 @@ int plan_gathered_count(sddmm_ctx *c, int min_fill, bool *launched) {
     c->n_cand = (int64_t)c->raw.n_candidates;
     if (c->n_cand < 2) { c->n_cand = 0; return SDDMM_OK; }
     int rc;
-    // candidates ordered by (first column, row)
-    size_t need = 0;
-    HIP_TRY(c, rocprim::radix_sort_keys(nullptr, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
-                                        c->stream));
-    if (need > c->sort_tmp_bytes) {
-        dfree(c->d_sort_tmp);
-        ALLOC_TRY(c, c->d_sort_tmp, need);
-        c->sort_tmp_bytes = need;
+    // candidates ordered by (first column, row): a few thousand by their ranks in one launch (4 us against 23 us
+    // for the radix sort on 3 000 keys), more by the library's radix sort
+    if (c->n_cand <= RANK_SORT_MAX && env_int("SDDMM_RANK_SORT", 1) != 0) {
+        constexpr int per_block = RANK_SORT_BLOCK / RANK_SORT_SPLIT;
+        SDDMM_LAUNCH(c, k_rank_sort, (unsigned)((c->n_cand + per_block - 1) / per_block), RANK_SORT_BLOCK,
+                           (const unsigned long long *)c->d_cand_keys, (unsigned long long *)c->d_sorted_keys, (int)c->n_cand);
+        LAUNCH_CHECK(c);
+    } else {
+        size_t need = 0;
+        HIP_TRY(c, rocprim::radix_sort_keys(nullptr, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
+                                            c->stream));
+        if (need > c->sort_tmp_bytes) {
+            dfree(c->d_sort_tmp);
+            ALLOC_TRY(c, c->d_sort_tmp, need);
+            c->sort_tmp_bytes = need;
+        }
+        HIP_TRY(c, rocprim::radix_sort_keys(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
+                                            c->stream));
     }
-    HIP_TRY(c, rocprim::radix_sort_keys(c->d_sort_tmp, need, c->d_cand_keys, c->d_sorted_keys, (size_t)c->n_cand, 0, 64,
-                                        c->stream));
     // pairs of strips: 32 consecutive candidates share one list of tile columns
     const int64_t n_vpairs = (c->n_cand + 31) / 32;
     c->n_vstrips = 2 * n_vpairs;
