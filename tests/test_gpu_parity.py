@@ -877,6 +877,13 @@ def test_gathered_pairs_behind_other_tiles(engine_factory, monkeypatch, K, dtype
     walk, st2 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
     assert st2.mfma_tiles == st.mfma_tiles
     assert_parity(walk, rowptr, col, val, A, B, what="pairs, tile by tile")
+    monkeypatch.delenv("SDDMM_WINDOW_FILL")
+    monkeypatch.delenv("SDDMM_PAIRS")
+    # the candidates ordered by the library's radix sort instead of by their ranks: the same plan, the same bits
+    monkeypatch.setenv("SDDMM_RANK_SORT", "0")
+    radix, st3 = run_csr(engine_factory, rowptr, col, val, *ops, N, capi.AUTO, dt)
+    assert st3.mfma_tiles == st.mfma_tiles and st3.nnz_mfma == st.nnz_mfma
+    np.testing.assert_array_equal(radix.view(np.uint32), got.view(np.uint32))
 
 
 def _host_union_model(M, rowptr, col, min_fill, span_limit=131072):
